@@ -15,6 +15,10 @@
 //   relu_sq            y = relu(x)^2
 //   glu_clamp          y = g' * sigmoid(alpha g') * (u' + bias),  g' = min(g, limit), u' = clamp(u, +-limit)
 //   group_topk         sigmoid scores -> best groups by the sum of their two largest -> top-k experts
+//   route_softmax      softmax scores (+ a selection bias) -> best groups by their largest biased score -> top-k;
+//                      trailing identity experts leave the pair list and come back as one gate per token
+//   rmsnorm_add        residual += rmsnorm(delta) * w;  y = residual (activation dtype)
+//   glu_act            silu(g) * u  or  gelu_tanh(g) * u  of  x = g | u
 //   gather_rows        xs[r] = x[idx[r]]
 //   moe_finish         residual[t] += sum_k w[t,k] * y[pos[t,k]] + gate[t] * shared[t]
 //
@@ -336,6 +340,118 @@ __global__ __launch_bounds__(64) void group_topk_kernel(const float* __restrict_
   }
 }
 
+// Softmax routing with a selection bias.  Scores s = softmax(z) over all n outputs; an expert is chosen by
+// c = s + bias, weighted by s.  Experts form `groups` equal runs of neighbours, a group scores its largest c and
+// only the `keep` best groups take part (the rest count as minus infinity; c may be negative).  The last
+// n - experts outputs are identity experts: a chosen one adds its score to gate[t] and leaves the pair list
+// (weight 0, id = park).  Ties go to the lower index.  One wave per token.
+__global__ __launch_bounds__(64) void route_softmax_kernel(const float* __restrict__ logits, int cols,
+                                                           const float* __restrict__ bias,
+                                                           float* __restrict__ weights, int* __restrict__ ids,
+                                                           float* __restrict__ gate, int n, int experts, int groups,
+                                                           int keep, int topk, float route_scale, int park) {
+  __shared__ float s[ROUTE_MAX_EXPERTS];
+  __shared__ float c[ROUTE_MAX_EXPERTS];
+  __shared__ float gs[ROUTE_MAX_EXPERTS];
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float* z = logits + t * cols;
+  float mx = -INFINITY;
+  for (int e = lane; e < n; e += 64) mx = fmaxf(mx, z[e]);
+  mx = wave_reduce_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < n; e += 64) {
+    const float v = expf(z[e] - mx);
+    s[e] = v;
+    sum += v;
+  }
+  sum = wave_reduce_sum(sum);
+  __syncthreads();
+  for (int e = lane; e < n; e += 64) {
+    const float v = s[e] / sum;
+    s[e] = v;
+    c[e] = v + (bias ? bias[e] : 0.f);
+  }
+  __syncthreads();
+  const int per = n / groups;
+  for (int g = lane; g < groups; g += 64) {
+    float a = -INFINITY;
+    for (int e = g * per; e < (g + 1) * per; ++e) a = fmaxf(a, c[e]);
+    gs[g] = a;
+  }
+  __syncthreads();
+  for (int g = lane; g < groups; g += 64) {
+    int ahead = 0;
+    const float v = gs[g];
+    for (int o = 0; o < groups; ++o) ahead += (gs[o] > v) || (gs[o] == v && o < g);
+    if (ahead >= keep)
+      for (int e = g * per; e < (g + 1) * per; ++e) c[e] = -INFINITY;
+  }
+  __syncthreads();
+  float gsum = 0.f;
+  for (int k = 0; k < topk; ++k) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < n; e += 64)
+      if (c[e] > best) { best = c[e]; bi = e; }
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, 64);
+      const int oi = __shfl_xor(bi, off, 64);
+      if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+    }
+    const bool none = bi == 0x7fffffff;  // fewer candidates than topk: an empty pair
+    if (lane == 0) {
+      const bool ident = !none && bi >= experts;
+      const float w = none ? 0.f : s[bi] * route_scale;
+      if (ident) gsum += w;
+      weights[t * topk + k] = (ident || none) ? 0.f : w;
+      ids[t * topk + k] = (ident || none) ? park : bi;
+    }
+    __syncthreads();
+    if (lane == 0 && !none) c[bi] = -INFINITY;
+    __syncthreads();
+  }
+  if (lane == 0 && gate) gate[t] = gsum;
+}
+
+// residual fp32 [rows, n] += rmsnorm(delta) * w (a norm on a sublayer's OUTPUT); y = the new residual, rounded
+template <typename T, typename D>
+__global__ __launch_bounds__(256) void rmsnorm_add_kernel(float* __restrict__ residual, const D* __restrict__ delta,
+                                                          long d_stride, const float* __restrict__ w,
+                                                          T* __restrict__ y, int n, float eps) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  float* r = residual + row * n;
+  const D* d = delta + row * d_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const float v = Conv<D>::ld(d + i);
+    ss += v * v;
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const float v = r[i] + Conv<D>::ld(d + i) * inv * w[i];
+    r[i] = v;
+    if (y) Conv<T>::st(y + row * n + i, v);
+  }
+}
+
+// x [rows, 2 inter] = gate | up  ->  act(gate) * up;  kind 0: silu, 1: gelu in its tanh form
+template <typename T>
+__global__ __launch_bounds__(256) void glu_act_kernel(const T* __restrict__ x, long x_stride, T* __restrict__ y,
+                                                      int inter, long total, int kind) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    const long row = i / inter;
+    const int col = (int)(i - row * inter);
+    const float g = Conv<T>::ld(x + row * x_stride + col);
+    const float u = Conv<T>::ld(x + row * x_stride + inter + col);
+    float a;
+    if (kind == 0) a = g * sigmoidf(g);
+    else a = 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    Conv<T>::st(y + i, a * u);
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const T* __restrict__ x, const int* __restrict__ idx,
                                                           T* __restrict__ xs, int n) {
@@ -479,6 +595,45 @@ VPSA_EXPORT int vpsa_group_topk(const float* logits, int cols, float* weights, i
     return -1;
   hipLaunchKernelGGL(group_topk_kernel, dim3(tokens), dim3(64), 0, st, logits, cols, weights, ids, extra_out,
                      experts, groups, keep, topk, route_scale);
+  return 0;
+}
+
+// park: the id a chosen identity expert's pair gets (its weight is 0): the expert count for callers that sort pairs
+// into a bucket no product visits, 0 for callers that run every pair.
+VPSA_EXPORT int vpsa_route_softmax(const float* logits, int cols, const float* bias, float* weights, int* ids,
+                                   float* gate, int tokens, int n, int experts, int groups, int keep, int topk,
+                                   float route_scale, int park, hipStream_t st) {
+  if (tokens <= 0) return 0;
+  if (n > ROUTE_MAX_EXPERTS || experts > n || groups < 1 || n % groups || keep < 1 || keep > groups || cols < n ||
+      topk < 1 || (experts < n && !gate))
+    return -1;
+  hipLaunchKernelGGL(route_softmax_kernel, dim3(tokens), dim3(64), 0, st, logits, cols, bias, weights, ids, gate, n,
+                     experts, groups, keep, topk, route_scale, park);
+  return 0;
+}
+
+// delta_f32: the delta is fp32 whatever the activation dtype (a mixture's fp32 sum)
+VPSA_EXPORT int vpsa_rmsnorm_add(float* residual, const void* delta, long d_stride, int delta_f32, const float* w,
+                                 void* y, int rows, int n, float eps, int dtype, hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (dtype != 0 && dtype != 1) return -2;
+  if (dtype == 1)
+    rmsnorm_add_kernel<float, float><<<rows, 256, 0, st>>>(residual, (const float*)delta, d_stride, w, (float*)y, n, eps);
+  else if (delta_f32)
+    rmsnorm_add_kernel<bf16_t, float><<<rows, 256, 0, st>>>(residual, (const float*)delta, d_stride, w, (bf16_t*)y, n, eps);
+  else
+    rmsnorm_add_kernel<bf16_t, bf16_t><<<rows, 256, 0, st>>>(residual, (const bf16_t*)delta, d_stride, w, (bf16_t*)y, n, eps);
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_glu_act(const void* x, long x_stride, void* y, int rows, int inter, int kind, int dtype,
+                             hipStream_t st) {
+  const long total = (long)rows * inter;
+  if (total <= 0) return 0;
+  if (kind < 0 || kind > 1) return -1;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(glu_act_kernel<bf16_t>, dim3(flat_grid(total)), dim3(256), 0, st, (const bf16_t*)x, x_stride, (bf16_t*)y, inter, total, kind),
+           hipLaunchKernelGGL(glu_act_kernel<float>, dim3(flat_grid(total)), dim3(256), 0, st, (const float*)x, x_stride, (float*)y, inter, total, kind));
   return 0;
 }
 

@@ -16,6 +16,16 @@
 //                      j <= i with i - j < window or j < keep_first, applied to the values of EVERY KV head
 //   mix_heads          out[t, h] = sum_g talk[h, g] u[t, g, kv_head(h)]
 //   xielu              z > 0: a_p z^2 + z / 2;  else a_n (exp(z) - 1 - z) + z / 2
+//   qk_norm_write      q and k heads to unit root mean square (no weight), q times a temperature that grows with
+//                      the logarithm of the position, k and v -> paged cache (the layout window_attention reads)
+//   gla_prepare        q scale | k | sigmoid(z + b)^(1 / tau) per key channel, for prepared_scan
+//   mlstm_gates        capped exponential input / forget gates of a matrix memory with their running maximum
+//                      (carried per sequence and head), turned into one decay and one write strength per token
+//   mlstm_prepare      q scale | k * write strength | decay, for prepared_scan
+//   prepared_scan      recurrent_scan on rows prepared by the caller; optionally one more value column of ones,
+//                      whose read-out is the normaliser's dot product with the query
+//   head_finish        head_rms with its parts optional: stabilised division by the normaliser column, unit RMS,
+//                      a weight per channel or per head and channel, a silu or sigmoid gate
 //
 // Plain kernels: every size is taken (bounds below are checked by the entry points).
 #include "common.h"
@@ -146,7 +156,9 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
     const T* __restrict__ proj, long p_stride, int v_col, int heads, int dim, int vdim, const float* __restrict__ prep,
     float* __restrict__ state, long state_stride, const int* __restrict__ seq_cu, const int* __restrict__ seq_state,
     const int* __restrict__ positions, const float* __restrict__ decay, float* __restrict__ out, int R, int TB,
-    const int* __restrict__ pieces, float* __restrict__ ws_state) {
+    const int* __restrict__ pieces, float* __restrict__ ws_state, int vsrc, int unit_col) {
+  // vsrc: value columns per head that `proj` holds (vdim, or one less than the state's columns need when
+  // unit_col: column vsrc of every token's value is then 1 and columns past it are 0)
   constexpr int NP = GATED ? 3 : 2;
   extern __shared__ float smem[];
   const int head = blockIdx.y;
@@ -220,7 +232,8 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
     for (int e = tid; e < nb * cols; e += 256) {
       const int tt = e / cols, c = e - tt * cols;
       const int cc = blockIdx.x * cols + c;
-      vs[e] = cc < vdim ? Cv<T>::ld(proj + (long)(rb + tt) * p_stride + v_col + head * vdim + cc) : 0.f;
+      vs[e] = cc < vsrc ? Cv<T>::ld(proj + (long)(rb + tt) * p_stride + v_col + head * vsrc + cc)
+                        : ((unit_col && cc == vsrc) ? 1.f : 0.f);
     }
     __syncthreads();
     for (int tt = 0; tt < nb; ++tt) {
@@ -333,27 +346,191 @@ __global__ __launch_bounds__(256) void scan_propagate_kernel(float* __restrict__
   *st = S;
 }
 
-// one wave per (row, head)
+// A piece's total decay per state row from prepared rows (prep [rows, heads, 3, dim], the third part).
+__global__ __launch_bounds__(128) void scan_decay_prep_kernel(const float* __restrict__ prep, int heads, int dim,
+                                                              const int* __restrict__ pieces,
+                                                              float* __restrict__ ws_decay) {
+  const int piece = blockIdx.x, head = blockIdx.y;
+  const int r0 = pieces[3 * piece + 1], n = pieces[3 * piece + 2];
+  for (int i = threadIdx.x; i < dim; i += 128) {
+    float p = 1.f;
+    for (int r = r0; r < r0 + n; ++r) p *= prep[((long)r * heads + head) * 3 * dim + 2 * dim + i];
+    ws_decay[((long)piece * heads + head) * dim + i] = p;
+  }
+}
+
+__device__ __forceinline__ float log_sigm(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
+
+// Gated linear attention: prep = q * q_scale | k | a,  a = sigmoid(z + b)^(1 / tau) per head and key channel.
 template <typename T>
-__global__ __launch_bounds__(256) void head_rms_kernel(const float* __restrict__ o, const float* __restrict__ w,
-                                                       const T* __restrict__ gate, long g_stride, T* __restrict__ y,
-                                                       long pairs, int heads, int vdim, float eps) {
+__global__ __launch_bounds__(256) void gla_prepare_kernel(const T* __restrict__ proj, long p_stride, int q_col, int k_col,
+                                                          const T* __restrict__ z, long z_stride,
+                                                          const float* __restrict__ z_bias, int heads, int dim,
+                                                          float q_scale, float inv_tau, float* __restrict__ prep) {
+  const long row = blockIdx.x;
+  const T* pr = proj + row * p_stride;
+  float* dst = prep + row * (long)heads * 3 * dim;
+  for (int e = threadIdx.x; e < heads * dim; e += 256) {
+    const int h = e / dim, i = e - h * dim;
+    float* d = dst + (long)h * 3 * dim + i;
+    d[0] = Cv<T>::ld(pr + q_col + e) * q_scale;
+    d[dim] = Cv<T>::ld(pr + k_col + e);
+    d[2 * dim] = expf(log_sigm(Cv<T>::ld(z + row * z_stride + e) + z_bias[e]) * inv_tau);
+  }
+}
+
+// Matrix memory with exponential gates.  Per head and token a log input gate i = cap tanh((x_i + b_i) / cap) and a
+// log forget gate f = logsigmoid(cap tanh((x_f + b_f) / cap)); a running maximum m_t = max(f_t + m_(t-1), i_t)
+// (m = 0 before the first token) keeps the exponentials in range:
+//   decay_t = exp(f_t + m_(t-1) - m_t),  write_t = exp(i_t - m_t).
+// The map m -> max(a + m, b) composes associatively, so a wave scans 64 tokens per step.  m is carried in the
+// sequence's state slot.  logits fp32 [rows, 2 heads] = x_i | x_f.  One wave per (sequence, head).
+__global__ __launch_bounds__(64) void mlstm_gates_kernel(const float* __restrict__ logits, const float* __restrict__ bias_i,
+                                                         const float* __restrict__ bias_f, float cap, int heads,
+                                                         float* __restrict__ state, long state_stride,
+                                                         const int* __restrict__ seq_cu,
+                                                         const int* __restrict__ seq_state,
+                                                         const int* __restrict__ positions, float* __restrict__ ab,
+                                                         float* __restrict__ mrow) {
+  const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int r0 = seq_cu[seq], r1 = seq_cu[seq + 1];
+  const int slot = seq_state[seq];
+  if (r1 <= r0) return;
+  if (slot < 0) {  // rows of no sequence: nothing is written into a state, the read-out is zero
+    for (int r = r0 + lane; r < r1; r += 64) {
+      ab[((long)r * heads + head) * 2] = 0.f;
+      ab[((long)r * heads + head) * 2 + 1] = 0.f;
+      mrow[(long)r * heads + head] = 0.f;
+    }
+    return;
+  }
+  float* mp = state + (long)slot * state_stride + head;
+  float m0 = positions[r0] == 0 ? 0.f : *mp;
+  const float bi = bias_i[head], bf = bias_f[head];
+  for (int rb = r0; rb < r1; rb += 64) {
+    const int r = rb + lane;
+    const bool live = r < r1;
+    float gi = -INFINITY, gf = 0.f;
+    if (live) {
+      gi = cap * tanhf((logits[(long)r * 2 * heads + head] + bi) / cap);
+      gf = log_sigm(cap * tanhf((logits[(long)r * 2 * heads + heads + head] + bf) / cap));
+    }
+    float a = gf, b = gi;  // this token's map, then the composition of all maps up to it
+    for (int off = 1; off < 64; off <<= 1) {
+      const float pa = __shfl_up(a, off, 64), pb = __shfl_up(b, off, 64);
+      if (lane >= off) {
+        b = fmaxf(pb + a, b);
+        a = pa + a;
+      }
+    }
+    const float m = fmaxf(a + m0, b);
+    float prev = __shfl_up(m, 1, 64);
+    if (lane == 0) prev = m0;
+    if (live) {
+      ab[((long)r * heads + head) * 2] = expf(gf + prev - m);
+      ab[((long)r * heads + head) * 2 + 1] = expf(gi - m);
+      mrow[(long)r * heads + head] = m;
+    }
+    m0 = __shfl(m, min(63, r1 - rb - 1), 64);
+  }
+  if (lane == 0) *mp = m0;
+}
+
+// prep = q * q_scale | k * write | decay (one decay for all key channels of a head)
+template <typename T>
+__global__ __launch_bounds__(256) void mlstm_prepare_kernel(const T* __restrict__ proj, long p_stride, int q_col,
+                                                            int k_col, const float* __restrict__ ab, int heads, int dim,
+                                                            float q_scale, float* __restrict__ prep) {
+  const long row = blockIdx.x;
+  const T* pr = proj + row * p_stride;
+  float* dst = prep + row * (long)heads * 3 * dim;
+  for (int e = threadIdx.x; e < heads * dim; e += 256) {
+    const int h = e / dim, i = e - h * dim;
+    float* d = dst + (long)h * 3 * dim + i;
+    const float dec = ab[(row * heads + h) * 2], wr = ab[(row * heads + h) * 2 + 1];
+    d[0] = Cv<T>::ld(pr + q_col + e) * q_scale;
+    d[dim] = Cv<T>::ld(pr + k_col + e) * wr;
+    d[2 * dim] = dec;
+  }
+}
+
+// One workgroup per row, a wave per head in turn.  Row = q [heads * dim] (| k [kv_heads * dim] | v [kv_heads * vdim]
+// when the layer owns its cache entries).  q and k heads are divided by their root mean square (eps inside the
+// root, no weight); q is then multiplied by 1 + coef ln(floor((p + 1) / every) + 1) at position p.  k and v go to
+// the page layout of window_attention (K key by key, V transposed).
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_write_kernel(const T* __restrict__ proj, long p_stride, int heads,
+                                                            int kv_heads, int dim, int vdim, int own,
+                                                            const int* __restrict__ positions,
+                                                            const long* __restrict__ slots, float eps, float coef,
+                                                            float every, T* __restrict__ q_out, T* __restrict__ cache,
+                                                            long page_stride) {
+  const long row = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* pr = proj + row * p_stride;
+  const int p = positions[row];
+  float temp = 1.f;
+  if (coef != 0.f) temp = 1.f + coef * logf((float)floor((double)(p + 1) / (double)every) + 1.f);
+  const long slot = own ? slots[row] : -1;
+  const int nk = kv_heads * dim;
+  for (int hh = wave; hh < heads + (own ? kv_heads : 0); hh += 4) {
+    const T* src = pr + (long)hh * dim;  // k heads follow the q heads
+    float ss = 0.f;
+    for (int i = lane; i < dim; i += 64) {
+      const float v = Cv<T>::ld(src + i);
+      ss += v * v;
+    }
+    ss = wave_reduce_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)dim + eps);
+    if (hh < heads) {
+      for (int i = lane; i < dim; i += 64) Cv<T>::st(q_out + (row * heads + hh) * dim + i, Cv<T>::ld(src + i) * inv * temp);
+    } else if (slot >= 0) {
+      T* dst = cache + (slot / PAGE) * page_stride + (slot % PAGE) * nk + (long)(hh - heads) * dim;
+      for (int i = lane; i < dim; i += 64) Cv<T>::st(dst + i, Cv<T>::ld(src + i) * inv);
+    }
+  }
+  if (slot >= 0) {
+    const T* vs = pr + (long)heads * dim + nk;
+    T* dst = cache + (slot / PAGE) * page_stride + (long)PAGE * nk + (slot % PAGE);
+    for (int c = threadIdx.x; c < kv_heads * vdim; c += 256) dst[(long)c * PAGE] = vs[c];
+  }
+}
+
+// One wave per (row, head).  o [pairs][ostride] fp32, of which the first vdim columns are the head's output.
+// stab: column vdim of o is the normaliser's dot product with the query and stab[pair] the running maximum m of the
+// gates: the output is first divided by max(|n . q|, exp(-m)) + 1e-6.  unit: divide by the root mean square over
+// vdim (eps inside the root).  w: a weight per channel (w_heads 0: shared by the heads) or per head and channel.
+// gate: times silu (gate_act 0) or sigmoid (1) of gate[row, head * vdim + c].
+template <typename T>
+__global__ __launch_bounds__(256) void head_rms_kernel(const float* __restrict__ o, int ostride,
+                                                       const float* __restrict__ stab, int unit,
+                                                       const float* __restrict__ w, int w_heads,
+                                                       const T* __restrict__ gate, long g_stride, int gate_act,
+                                                       T* __restrict__ y, long pairs, int heads, int vdim, float eps) {
   const long pair = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (pair >= pairs) return;
   const int lane = threadIdx.x & 63;
   const long row = pair / heads;
   const int head = (int)(pair - row * heads);
-  const float* op = o + pair * vdim;
-  float ss = 0.f;
-  for (int c = lane; c < vdim; c += 64) ss += op[c] * op[c];
-  ss = wave_reduce_sum(ss);
-  const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
+  const float* op = o + pair * ostride;
+  float pre = 1.f;
+  if (stab) pre = 1.f / (fmaxf(fabsf(op[vdim]), expf(-stab[pair])) + 1e-6f);
+  float inv = 1.f;
+  if (unit) {
+    float ss = 0.f;
+    for (int c = lane; c < vdim; c += 64) {
+      const float v = op[c] * pre;
+      ss += v * v;
+    }
+    ss = wave_reduce_sum(ss);
+    inv = 1.f / sqrtf(ss / (float)vdim + eps);
+  }
   for (int c = lane; c < vdim; c += 64) {
-    float v = op[c] * inv;
-    if (w) v *= w[c];
+    float v = op[c] * pre * inv;
+    if (w) v *= w[w_heads ? head * vdim + c : c];
     if (gate) {
       const float g = Cv<T>::ld(gate + row * g_stride + head * vdim + c);
-      v *= g * sigm(g);
+      v *= gate_act == 0 ? g * sigm(g) : sigm(g);
     }
     Cv<T>::st(y + pair * vdim + c, v);
   }
@@ -466,7 +643,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
     const T* __restrict__ q, long q_stride, const T* __restrict__ cache, long page_stride,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ row_seq,
     const int* __restrict__ positions, const float* __restrict__ sink, float* __restrict__ out, int heads, int kv_heads,
-    int dim, int vdim, int window, int keep_first, float scale, float softcap) {
+    int dim, int vdim, int window, int keep_first, float scale, float softcap, int own) {
+  // own: only the values of the head's own KV head (out [rows, heads, vdim]); designs without head mixing
   extern __shared__ float sm[];
   __shared__ float red[4];
   __shared__ float ps[WA_KEYS];
@@ -478,7 +656,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
   const int seq = row_seq ? row_seq[row] : (int)row;
   const int pos = positions[row];
   const int g = head / (heads / kv_heads);
-  const int nk = kv_heads * dim, nv = kv_heads * vdim;
+  const int nk = kv_heads * dim, nv = own ? vdim : kv_heads * vdim;
+  const int c0 = own ? g * vdim : 0;  // first value channel this head reads
   float* qs = sm;
   for (int i = tid; i < dim; i += 256) qs[i] = Cv<T>::ld(q + row * q_stride + head * dim + i);
   const PageWalk walk(pos, pos, window, keep_first);
@@ -519,7 +698,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
       if (c < nv) {
         float x = acc[a] * corr;
         for (int pp = 0; pp < np; ++pp) {
-          const T* vp = cache + pbase[pp] + (long)PAGE * nk + (long)c * PAGE;
+          const T* vp = cache + pbase[pp] + (long)PAGE * nk + (long)(c0 + c) * PAGE;
           for (int k = 0; k < PAGE; k += RUN) {
             T v[RUN];
             *reinterpret_cast<u32x4*>(v) = *reinterpret_cast<const u32x4*>(vp + k);
@@ -558,7 +737,9 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles,
     const int* __restrict__ positions, const float* __restrict__ sink, float* __restrict__ out, int heads, int kv_heads,
     int window, int keep_first, float scale, float softcap, int splits, float* __restrict__ ws_o,
-    float* __restrict__ ws_ml, int n_chunks) {
+    float* __restrict__ ws_ml, int n_chunks, int own) {
+  // own: a slot's weights meet the values of its own KV head only (n_chunks chunks of VALL channels per KV head,
+  // out [rows, heads, n_chunks * VALL]); else those of every KV head (n_chunks chunks over all of them)
   constexpr int KS = DIM / 32;
   constexpr int DT = VALL / 16;
   constexpr int PK = DIM * 2 + 16;
@@ -632,7 +813,8 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     }
 #pragma unroll
     for (int b = 0; b < VB; ++b)
-      vb[b] = *reinterpret_cast<const u32x4*>(src + v_off + (long)chunk * VALL * PAGE + (long)(tid + 256 * b) * 8);
+      vb[b] = *reinterpret_cast<const u32x4*>(src + v_off + (long)(own ? group * n_chunks + chunk : chunk) * VALL * PAGE +
+                                              (long)(tid + 256 * b) * 8);
   };
   auto stash = [&]() {
 #pragma unroll
@@ -865,13 +1047,15 @@ static void scan_shape(int dim, int* rpt, int* r) {
 // ws_state fp32 [n_pieces, heads, dim, vdim], ws_decay fp32 [n_pieces, heads, dim].  prep: fp32 workspace
 // [rows, heads, 2 (3 when gated), dim].  fold: every decay's 16th power is well inside fp32's range (the kernel
 // then folds the decay into the staged keys and queries).
-VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, int k_col, int v_col, int heads, int dim,
-                                    int vdim, float* state, long state_stride, const int* seq_cu, const int* seq_state,
-                                    int n_seqs, const int* positions, const float* decay, const float* cos_sin,
-                                    int rot_dims, int layout, float k_scale, const float* gate_bias,
-                                    const float* gate_lower, float* out, int gated, const int* pieces,
-                                    const int* seq_pieces, int n_pieces, float* ws_state, float* ws_decay, float* prep,
-                                    int rows, int fold, int dt, hipStream_t stream) {
+// prepared: `prep` already holds q' | k' | a for every row (the caller's own gates): nothing is prepared here, the
+// pieces' decays come from it, and `proj` only serves the values (vsrc columns per head; with unit_col the state has
+// one more column, fed with ones).
+static int scan_run(const void* proj, long p_stride, int q_col, int k_col, int v_col, int heads, int dim, int vdim,
+                    float* state, long state_stride, const int* seq_cu, const int* seq_state, int n_seqs,
+                    const int* positions, const float* decay, const float* cos_sin, int rot_dims, int layout,
+                    float k_scale, const float* gate_bias, const float* gate_lower, float* out, int gated,
+                    const int* pieces, const int* seq_pieces, int n_pieces, float* ws_state, float* ws_decay,
+                    float* prep, int rows, int fold, int dt, hipStream_t stream, int prepared, int vsrc, int unit_col) {
   if (n_seqs <= 0 || rows <= 0) return 0;
   int rpt, r;
   scan_shape(dim, &rpt, &r);
@@ -886,7 +1070,7 @@ VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, 
 #define SCAN(RPT, G, F, PH, NZ)                                                                                        \
   recurrent_scan_kernel<T, RPT, G, F, PH><<<dim3(col_blocks, heads, NZ), 256, lds, stream>>>(                          \
       (const T*)proj, p_stride, v_col, heads, dim, vdim, prep, state, state_stride, seq_cu, seq_state, positions,     \
-      decay, out, r, tb, pieces, ws_state)
+      decay, out, r, tb, pieces, ws_state, vsrc, unit_col)
 #define SCAN_R(G, F, PH, NZ)                       \
   if (rpt == 8) SCAN(8, G, F, PH, NZ);             \
   else if (rpt == 16) SCAN(16, G, F, PH, NZ);      \
@@ -895,7 +1079,8 @@ VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, 
   if (gated) { SCAN_R(true, false, PH, NZ) }       \
   else if (fold) { SCAN_R(false, true, PH, NZ) }   \
   else { SCAN_R(false, false, PH, NZ) }
-  if (gated) {
+  if (prepared) {
+  } else if (gated) {
     SM_DISPATCH(dt, (scan_prepare_kernel<T, true><<<rows, 256, 0, stream>>>((const T*)proj, p_stride, q_col, k_col, heads,
                                                                             dim, positions, cos_sin, rot_dims, layout,
                                                                             k_scale, gate_bias, gate_lower, prep)));
@@ -909,7 +1094,9 @@ VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, 
     return 0;
   }
   if (n_pieces <= 0 || !seq_pieces || !ws_state || !ws_decay) return 4;
-  if (gated) {
+  if (prepared) {
+    scan_decay_prep_kernel<<<dim3(n_pieces, heads), 128, 0, stream>>>(prep, heads, dim, pieces, ws_decay);
+  } else if (gated) {
     SM_DISPATCH(dt, (scan_decay_kernel<T, true><<<dim3(n_pieces, heads), 128, 0, stream>>>(
                         (const T*)proj, p_stride, k_col, heads, dim, decay, gate_bias, gate_lower, pieces, ws_decay)));
   } else {
@@ -926,12 +1113,84 @@ VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, 
   return 0;
 }
 
-VPSA_EXPORT int vpsa_head_rms(const float* o, const float* w, const void* gate, long g_stride, void* y, int rows,
-                              int heads, int vdim, float eps, int dt, hipStream_t stream) {
+VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, int k_col, int v_col, int heads, int dim,
+                                    int vdim, float* state, long state_stride, const int* seq_cu, const int* seq_state,
+                                    int n_seqs, const int* positions, const float* decay, const float* cos_sin,
+                                    int rot_dims, int layout, float k_scale, const float* gate_bias,
+                                    const float* gate_lower, float* out, int gated, const int* pieces,
+                                    const int* seq_pieces, int n_pieces, float* ws_state, float* ws_decay, float* prep,
+                                    int rows, int fold, int dt, hipStream_t stream) {
+  return scan_run(proj, p_stride, q_col, k_col, v_col, heads, dim, vdim, state, state_stride, seq_cu, seq_state, n_seqs,
+                  positions, decay, cos_sin, rot_dims, layout, k_scale, gate_bias, gate_lower, out, gated, pieces,
+                  seq_pieces, n_pieces, ws_state, ws_decay, prep, rows, fold, dt, stream, 0, vdim, 0);
+}
+
+// The recurrence over rows the caller prepared: prep fp32 [rows, heads, 3, dim] = q' | k' | a, values from `v`
+// (row stride v_stride, heads side by side from column v_col, vsrc columns each).  The state has vdim columns per
+// key channel: vsrc, or with unit_col at least vsrc + 1 (column vsrc accumulates k' alone: read out by q' it is the
+// normaliser's dot product).  out fp32 [rows, heads, vdim].
+VPSA_EXPORT int vpsa_prepared_scan(const void* v, long v_stride, int v_col, int vsrc, int unit_col, int heads, int dim,
+                                   int vdim, float* prep, float* state, long state_stride, const int* seq_cu,
+                                   const int* seq_state, int n_seqs, const int* positions, float* out,
+                                   const int* pieces, const int* seq_pieces, int n_pieces, float* ws_state,
+                                   float* ws_decay, int rows, int dt, hipStream_t stream) {
+  if (vsrc + (unit_col ? 1 : 0) > vdim) return 5;
+  return scan_run(v, v_stride, 0, 0, v_col, heads, dim, vdim, state, state_stride, seq_cu, seq_state, n_seqs, positions,
+                  nullptr, nullptr, 0, 0, 1.f, nullptr, nullptr, out, 1, pieces, seq_pieces, n_pieces, ws_state,
+                  ws_decay, prep, rows, 0, dt, stream, 1, vsrc, unit_col);
+}
+
+VPSA_EXPORT int vpsa_gla_prepare(const void* proj, long p_stride, int q_col, int k_col, const void* z, long z_stride,
+                                 const float* z_bias, int heads, int dim, float q_scale, float tau, float* prep,
+                                 int rows, int dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  SM_DISPATCH(dt, (gla_prepare_kernel<T><<<rows, 256, 0, stream>>>((const T*)proj, p_stride, q_col, k_col, (const T*)z,
+                                                                   z_stride, z_bias, heads, dim, q_scale, 1.f / tau, prep)));
+  return 0;
+}
+
+// logits fp32 [rows, 2 heads] = input-gate | forget-gate pre-activations (without their biases); m_state: the
+// running maxima's place in the state pool (heads floats per slot).  Leaves prep (q * q_scale | k * write | decay)
+// and mrow fp32 [rows, heads] (the running maximum after every token); ab fp32 [rows, heads, 2] is workspace.
+VPSA_EXPORT int vpsa_mlstm_prepare(const void* proj, long p_stride, int q_col, int k_col, const float* logits,
+                                   const float* bias_i, const float* bias_f, float cap, int heads, int dim,
+                                   float q_scale, float* m_state, long state_stride, const int* seq_cu,
+                                   const int* seq_state, int n_seqs, const int* positions, float* ab, float* mrow,
+                                   float* prep, int rows, int dt, hipStream_t stream) {
+  if (rows <= 0 || n_seqs <= 0) return 0;
+  mlstm_gates_kernel<<<dim3(n_seqs, heads), 64, 0, stream>>>(logits, bias_i, bias_f, cap, heads, m_state, state_stride,
+                                                            seq_cu, seq_state, positions, ab, mrow);
+  SM_DISPATCH(dt, (mlstm_prepare_kernel<T><<<rows, 256, 0, stream>>>((const T*)proj, p_stride, q_col, k_col, ab, heads,
+                                                                     dim, q_scale, prep)));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_head_finish(const float* o, int ostride, const float* stab, int unit, const float* w, int w_heads,
+                                 const void* gate, long g_stride, int gate_act, void* y, int rows, int heads, int vdim,
+                                 float eps, int dt, hipStream_t stream) {
   const long pairs = (long)rows * heads;
   if (pairs <= 0) return 0;
-  SM_DISPATCH(dt, (head_rms_kernel<T><<<(unsigned)((pairs + 3) / 4), 256, 0, stream>>>(o, w, (const T*)gate, g_stride,
-                                                                                       (T*)y, pairs, heads, vdim, eps)));
+  if (ostride < vdim + (stab ? 1 : 0)) return 2;
+  SM_DISPATCH(dt, (head_rms_kernel<T><<<(unsigned)((pairs + 3) / 4), 256, 0, stream>>>(
+                      o, ostride, stab, unit, w, w_heads, (const T*)gate, g_stride, gate_act, (T*)y, pairs, heads, vdim,
+                      eps)));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_head_rms(const float* o, const float* w, const void* gate, long g_stride, void* y, int rows,
+                              int heads, int vdim, float eps, int dt, hipStream_t stream) {
+  return vpsa_head_finish(o, vdim, nullptr, 1, w, 0, gate, g_stride, 0, y, rows, heads, vdim, eps, dt, stream);
+}
+
+// proj rows: q | k | v when own (the layer caches its keys and values), q alone otherwise.
+VPSA_EXPORT int vpsa_qk_norm_write(const void* proj, long p_stride, int heads, int kv_heads, int dim, int vdim, int own,
+                                   const int* positions, const long* slots, float eps, float coef, float every,
+                                   void* q_out, void* cache, long page_stride, int rows, int dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (coef != 0.f && !(every > 0.f)) return 2;
+  SM_DISPATCH(dt, (qk_norm_write_kernel<T><<<rows, 256, 0, stream>>>((const T*)proj, p_stride, heads, kv_heads, dim, vdim,
+                                                                     own, positions, slots, eps, coef, every, (T*)q_out,
+                                                                     (T*)cache, page_stride)));
   return 0;
 }
 
@@ -957,14 +1216,14 @@ VPSA_EXPORT int vpsa_short_conv_qkv(const void* proj, long p_stride, const float
 VPSA_EXPORT int vpsa_window_attention(const void* q, long q_stride, const void* cache, long page_stride,
                                       const int* block_tables, int bt_stride, const int* row_seq, const int* positions,
                                       const float* sink, float* out, int rows, int heads, int kv_heads, int dim, int vdim,
-                                      int window, int keep_first, float scale, float softcap, int dt,
+                                      int window, int keep_first, float scale, float softcap, int own, int dt,
                                       hipStream_t stream) {
   if (rows <= 0) return 0;
-  if (kv_heads * vdim > 256 * WA_ACC || (size_t)dim * 4 > 32 * 1024) return 2;
+  if ((own ? vdim : kv_heads * vdim) > 256 * WA_ACC || (size_t)dim * 4 > 32 * 1024 || heads % kv_heads) return 2;
   dim3 grid(rows, heads);
   SM_DISPATCH(dt, (window_attention_kernel<T><<<grid, 256, (size_t)dim * 4, stream>>>(
                       (const T*)q, q_stride, (const T*)cache, page_stride, block_tables, bt_stride, row_seq, positions,
-                      sink, out, heads, kv_heads, dim, vdim, window, keep_first, scale, softcap)));
+                      sink, out, heads, kv_heads, dim, vdim, window, keep_first, scale, softcap, own)));
   return 0;
 }
 
@@ -975,8 +1234,8 @@ static int window_chunk(int vall) {
   return 0;
 }
 
-VPSA_EXPORT int vpsa_window_mfma_supported(int heads, int kv_heads, int dim, int vdim) {
-  return (dim == 64 || dim == 128) && window_chunk(kv_heads * vdim) > 0 && heads % kv_heads == 0 &&
+VPSA_EXPORT int vpsa_window_mfma_supported(int heads, int kv_heads, int dim, int vdim, int own) {
+  return (dim == 64 || dim == 128) && window_chunk(own ? vdim : kv_heads * vdim) > 0 && heads % kv_heads == 0 &&
          heads / kv_heads <= 64;
 }
 
@@ -989,7 +1248,8 @@ template <int DIM, int VALL, int NSUB>
 static int launch_window_mfma(const void* q, long q_stride, const void* cache, long page_stride, const int* block_tables,
                               int bt_stride, const int* tiles, const int* positions, const float* sink, float* out,
                               int n_tiles, int heads, int kv_heads, int window, int keep_first, float scale,
-                              float softcap, int splits, float* ws_o, float* ws_ml, int n_chunks, hipStream_t st) {
+                              float softcap, int splits, float* ws_o, float* ws_ml, int n_chunks, int own,
+                              hipStream_t st) {
   constexpr int LDS = PAGE * (DIM * 2 + 16) + VALL * (PAGE * 2 + 16);
   static bool attr_set = false;
   if (!attr_set) {
@@ -1000,7 +1260,7 @@ static int launch_window_mfma(const void* q, long q_stride, const void* cache, l
   }
   window_mfma_kernel<DIM, VALL, NSUB><<<dim3(n_tiles, kv_heads * n_chunks, splits), dim3(256), LDS, st>>>(
       (const uint16_t*)q, q_stride, (const uint16_t*)cache, page_stride, block_tables, bt_stride, tiles, positions, sink,
-      out, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o, ws_ml, n_chunks);
+      out, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o, ws_ml, n_chunks, own);
   if (splits > 1)  // decode rows only: row r of the launch is row r of out
     window_merge_kernel<<<n_tiles * heads, 128, 0, st>>>(ws_o, ws_ml, sink, out, heads, VALL * n_chunks, splits);
   return 0;
@@ -1015,21 +1275,22 @@ VPSA_EXPORT int vpsa_window_attention_mfma(const void* q, long q_stride, const v
                                            const int* block_tables, int bt_stride, const int* tiles,
                                            const int* positions, const float* sink, float* out, int n_tiles, int heads,
                                            int kv_heads, int dim, int vdim, int window, int keep_first, float scale,
-                                           float softcap, int splits, float* ws_o, float* ws_ml, hipStream_t stream) {
+                                           float softcap, int splits, float* ws_o, float* ws_ml, int own,
+                                           hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  if (!vpsa_window_mfma_supported(heads, kv_heads, dim, vdim)) return 2;
+  if (!vpsa_window_mfma_supported(heads, kv_heads, dim, vdim, own)) return 2;
   if (splits < 1 || (splits > 1 && (tiles || !ws_o || !ws_ml))) return 3;  // splits are for decode rows
-  const int vall = window_chunk(kv_heads * vdim), n_chunks = kv_heads * vdim / vall;
+  const int vall = window_chunk(own ? vdim : kv_heads * vdim), n_chunks = (own ? vdim : kv_heads * vdim) / vall;
 #define WM(D, V)                                                                                                      \
   if (dim == D && vall == V) {                                                                                        \
     if (tiles)                                                                                                        \
       return launch_window_mfma<D, V, WINDOW_PREFILL_SUB>(q, q_stride, cache, page_stride, block_tables, bt_stride,    \
                                                           tiles, positions, sink, out, n_tiles, heads, kv_heads,      \
                                                           window, keep_first, scale, softcap, splits, ws_o, ws_ml,     \
-                                                          n_chunks, stream);                                          \
+                                                          n_chunks, own, stream);                                     \
     return launch_window_mfma<D, V, 1>(q, q_stride, cache, page_stride, block_tables, bt_stride, tiles, positions,     \
                                        sink, out, n_tiles, heads, kv_heads, window, keep_first, scale, softcap,       \
-                                       splits, ws_o, ws_ml, n_chunks, stream);                                        \
+                                       splits, ws_o, ws_ml, n_chunks, own, stream);                                   \
   }
   WM(64, 128) WM(64, 256) WM(64, 512) WM(128, 128) WM(128, 256) WM(128, 512)
 #undef WM

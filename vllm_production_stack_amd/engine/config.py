@@ -53,7 +53,11 @@ class FeedForwardSpec:
     an always-on shared unit of width ``shared_ff`` (0 = none) with a per-token sigmoid gate."""
     kind: str = "dense"
     ff: int = 0
-    act: str = "relu_sq"       # dense units: relu_sq | xielu (two learned curvatures, see ops.xielu)
+    act: str = "relu_sq"       # relu_sq | xielu (two learned curvatures, see ops.xielu) | gelu_tanh | silu (gated units)
+    gated: bool = False        # down(act(gate x) * (up x)) instead of down(act(up x))
+    router: str = "sigmoid"    # sigmoid: as described above | softmax: softmax scores, a learned selection bias,
+                               # a group scores its largest biased score, weights = scores, not renormalised
+    identity: int = 0          # softmax router: extra outputs whose "expert" returns the token itself
     experts: int = 0
     top: int = 0
     groups: int = 1
@@ -173,6 +177,133 @@ class ParallelMixerSpec:
         return self.left.weight_count(width) + self.right.weight_count(width)
 
 
+@dataclass(frozen=True)
+class NormedAttentionSpec:
+    """Grouped-query softmax attention without rotation: q and k heads are divided by their root mean
+    square (no weight), q grows with the position by 1 + temp_coef ln(floor((p + 1) / temp_every) + 1),
+    a per-head sink logit joins the denominator, head outputs are gated by sigmoid(W_g h).  ``kv_from``:
+    the layer whose cached keys and values this layer reads instead of projecting its own."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    temp_coef: float = 0.0
+    temp_every: float = 1.0
+    kv_from: int | None = None
+
+    def cache_elems(self) -> int:        # per token, for layers that own their entries
+        return self.kv_heads * (self.dim + self.vdim) if self.kv_from is None else 0
+
+    def weight_count(self, width: int) -> int:
+        n = width * self.heads * (self.dim + self.vdim) + self.heads * self.vdim * width
+        return n + (width * self.kv_heads * (self.dim + self.vdim) if self.kv_from is None else 0)
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """A matrix memory with exponential gates: per head S <- exp(f + m' - m) S + exp(i - m) k v^T with a running
+    maximum m of the log gates, a normaliser n updated like S with k alone, o = S^T q / (max(|n . q|, exp(-m)) + 1e-6);
+    log gates i = cap tanh(. / cap), f = logsigmoid(cap tanh(. / cap)); heads brought to unit RMS, weighted
+    and gated by sigmoid(W_g h)."""
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+
+    def weight_count(self, width: int) -> int:
+        return width * self.heads * (2 * self.dim + 2 * self.vdim + 2) + self.heads * self.vdim * width
+
+    def token_flops(self) -> float:
+        return 4.0 * self.heads * self.dim * (self.vdim + 1)
+
+
+@dataclass(frozen=True)
+class GatedLinearSpec:
+    """Linear attention with a decay per key channel: S <- diag(a) S + k v^T, a = sigmoid(W_a2 W_a1 h + b)^(1 / tau)
+    through a low-rank pair of projections (``decay_rank``; a checkpoint's tensors decide it); heads RMS-normed
+    with one weight vector and gated by silu(W_g h)."""
+    heads: int
+    dim: int
+    vdim: int
+    tau: float
+    decay_rank: int = 16
+
+    def weight_count(self, width: int) -> int:
+        n = width * self.heads * (2 * self.dim + 2 * self.vdim) + self.heads * self.vdim * width
+        return n + self.decay_rank * (width + self.heads * self.dim)
+
+    def token_flops(self) -> float:
+        return 4.0 * self.heads * self.dim * self.vdim
+
+
+def pelatar_layers(layers: list[dict]) -> tuple:
+    """The ``layers`` list of a Pelatar config.json -> layer specs."""
+    out = []
+    for i, entry in enumerate(layers):
+        m = entry["mixer"]
+        kind = entry["type"]
+        if kind == "attention":
+            temp = m.get("q_temp") or {}
+            src = m.get("kv_from")
+            mixer = NormedAttentionSpec(
+                heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                scale=float(m["scale"]), temp_coef=float(temp.get("coef", 0.0)), temp_every=float(temp.get("every", 1.0)),
+                kv_from=None if src is None else int(src))
+            if mixer.heads % mixer.kv_heads or (mixer.temp_coef != 0.0 and mixer.temp_every <= 0):
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads and the temperature's period positive")
+            if mixer.kv_from is not None:
+                if not 0 <= mixer.kv_from < i:
+                    raise ValueError(f"layer {i}: kv_from must name an earlier layer")
+                s = out[mixer.kv_from].mixer
+                if (not isinstance(s, NormedAttentionSpec) or s.kv_from is not None
+                        or (s.kv_heads, s.dim, s.vdim) != (mixer.kv_heads, mixer.dim, mixer.vdim)):
+                    raise ValueError(f"layer {i}: layer {mixer.kv_from} does not hold keys and values of this layer's shape")
+        elif kind == "mlstm":
+            mixer = MatrixMemorySpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), float(m["gate_cap"]))
+            if mixer.gate_cap <= 0:
+                raise ValueError(f"layer {i}: gate_cap must be positive")
+        elif kind == "gla":
+            mixer = GatedLinearSpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), float(m["tau"]),
+                                    int(m.get("decay_rank", 16)))
+            if mixer.tau <= 0:
+                raise ValueError(f"layer {i}: tau must be positive")
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        f = entry.get("mlp")
+        mlp = None
+        if f is not None:
+            if f["kind"] == "dense":
+                mlp = FeedForwardSpec(kind="dense", ff=int(f["ff"]), act="gelu_tanh", gated=True)
+            elif f["kind"] == "moe":
+                r = f["router"]
+                g = r.get("groups") or {}
+                ident = int(r.get("identity", 0))
+                mlp = FeedForwardSpec(kind="moe", ff=int(f["expert"]["ff"]), act="silu", gated=True, experts=int(r["experts"]),
+                                      top=int(r["top"]), groups=int(g.get("count", 1)),
+                                      keep=int(g.get("keep", g.get("count", 1))), router="softmax", identity=ident)
+                n = mlp.experts + ident
+                if mlp.groups < 1 or n % mlp.groups or not 1 <= mlp.keep <= mlp.groups or mlp.top > n // mlp.groups * mlp.keep:
+                    raise ValueError(f"layer {i}: experts and identity experts must split into equal groups that hold `top`")
+            else:
+                raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+        out.append(LayerSpec(kind, mixer, mlp))
+    return tuple(out)
+
+
+def pelatar_config(name: str, vocab: int, width: int, layers: list[dict], norm_eps: float = 1e-5,
+                   max_position_embeddings: int = 32768) -> "ModelConfig":
+    specs = pelatar_layers(layers)
+    att = [s.mixer for s in specs if isinstance(s.mixer, NormedAttentionSpec)]
+    return ModelConfig(
+        name=name, architecture="pelatar", vocab_size=int(vocab), hidden_size=int(width),
+        intermediate_size=max([s.mlp.ff for s in specs if s.mlp] + [0]), num_layers=len(specs),
+        num_heads=max(s.mixer.heads for s in specs), num_kv_heads=max([a.kv_heads for a in att] + [1]),
+        head_dim=max(s.mixer.dim for s in specs), norm_eps=float(norm_eps),
+        max_position_embeddings=max_position_embeddings, tie_word_embeddings=True, layer_specs=specs,
+        bos_token_id=0, eos_token_id=-1)  # the design names no special tokens
+
+
 def _rotary(rot: dict, layout: str) -> RotarySpec:
     sc = rot.get("scaling")
     scaling = None if not sc else (float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"]))
@@ -284,7 +415,7 @@ def zururax_config(name: str, vocab: int, width: int, layers: list[dict], embedd
 @dataclass
 class ModelConfig:
     name: str = "tiny-llama"
-    architecture: str = "llama"  # llama | mixtral | opt | gpt2 | zururax | revelix
+    architecture: str = "llama"  # llama | mixtral | opt | gpt2 | zururax | revelix | pelatar
     vocab_size: int = 512
     hidden_size: int = 256
     intermediate_size: int = 512
@@ -330,6 +461,8 @@ class ModelConfig:
                 gemm += m.weight_count(h)
                 if isinstance(m, LatentMixerSpec):
                     pair += m.heads * (m.entry + m.kv_rank)
+                elif isinstance(m, NormedAttentionSpec):
+                    pair += m.heads * (m.dim + m.vdim)
                 else:  # recurrences cost per token, a windowed softmax at most its window per token
                     for part in (getattr(m, "left", None), getattr(m, "right", None), m):
                         if hasattr(part, "token_flops"):
@@ -337,7 +470,8 @@ class ModelConfig:
                         if isinstance(part, WindowAttentionSpec):
                             gemm += part.heads * (part.dim + part.kv_heads * part.vdim) * (part.window + part.keep_first)
                 if f is not None:
-                    gemm += 2 * h * f.ff if f.kind == "dense" else 3 * h * (f.top * f.ff + f.shared_ff) + h * f.experts
+                    gemm += ((3 if f.gated else 2) * h * f.ff if f.kind == "dense"
+                             else 3 * h * (f.top * f.ff + f.shared_ff) + h * (f.experts + f.identity))
             return 2.0 * gemm, 2.0 * pair
         attn_w = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         mlp_w = 3 * h * i * max(1, self.num_experts_per_tok if self.num_experts else 1)
@@ -351,7 +485,8 @@ class ModelConfig:
                 m, f = s.mixer, s.mlp
                 n += m.weight_count(h)
                 if f is not None:
-                    n += 2 * h * f.ff if f.kind == "dense" else 3 * h * (f.experts * f.ff + f.shared_ff) + h * f.experts
+                    n += ((3 if f.gated else 2) * h * f.ff if f.kind == "dense"
+                          else 3 * h * (f.experts * f.ff + f.shared_ff) + h * (f.experts + f.identity))
             return n
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         mlp = 3 * h * i * max(1, self.num_experts)
@@ -548,6 +683,10 @@ def _from_hf_config(cfg: dict[str, Any], name: str) -> ModelConfig:
     if str(cfg.get("architecture", "")).lower() == "revelix":
         return revelix_config(name, cfg["vocab"], cfg["width"], cfg["layers"], logit_scale=cfg.get("logit_scale", 1.0),
                               norm_eps=(cfg.get("norm") or {}).get("eps", 1e-6),
+                              max_position_embeddings=int(cfg.get("max_positions", 32768)))
+    if str(cfg.get("architecture", "")).lower() == "pelatar":
+        return pelatar_config(name, cfg["vocab"], cfg["width"], cfg["layers"],
+                              norm_eps=(cfg.get("norm") or {}).get("eps", 1e-5),
                               max_position_embeddings=int(cfg.get("max_positions", 32768)))
     arch = (cfg.get("architectures") or [""])[0].lower()
     mt = cfg.get("model_type", "").lower()

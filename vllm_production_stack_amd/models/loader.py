@@ -17,6 +17,7 @@ from ..engine.config import ModelConfig
 from ..parallel.state import get_tp
 from .opt import OPTModel
 from .transformer import LayerWeights, TransformerModel
+from .pelatar import PelatarModel
 from .revelix import RevelixModel
 from .zururax import ZururaxModel
 
@@ -30,6 +31,8 @@ def build_model(cfg: ModelConfig, dtype: torch.dtype, device: torch.device, max_
         model = ZururaxModel(cfg, dtype, device, max_model_len)
     elif cfg.architecture == "revelix":
         model = RevelixModel(cfg, dtype, device, max_model_len)
+    elif cfg.architecture == "pelatar":
+        model = PelatarModel(cfg, dtype, device, max_model_len)
     else:
         model = TransformerModel(cfg, dtype, device, max_model_len, expert_parallel=expert_parallel)
     has_weights = ckpt_dir is not None and any(Path(ckpt_dir).glob("*.safetensors"))
@@ -63,6 +66,8 @@ def load_hf_weights(model, ckpt_dir: Path) -> None:
         _load_zururax(model, ckpt_dir)
     elif isinstance(model, RevelixModel):
         _load_revelix(model, ckpt_dir)
+    elif isinstance(model, PelatarModel):
+        _load_pelatar(model, ckpt_dir)
     else:
         _load_llama(model, ckpt_dir)
 
@@ -458,5 +463,127 @@ def _load_revelix(model: RevelixModel, ckpt_dir: Path) -> None:
         if f is not None:
             want |= {f"l{i}.norm2{x}" for x in ("", ".b", ".alpha")}
             want |= {f"l{i}.mlp.{k}" for k in ("up", "down", "act")}
+    if want - seen:
+        raise ValueError(f"checkpoint lacks {sorted(want - seen)[:8]}")
+
+
+def _load_pelatar(model: PelatarModel, ckpt_dir: Path) -> None:
+    """Pelatar checkpoints: ``embed``; per layer ``l<i>.norm1|norm2``; ``l<i>.mix.{q, k, v, sink, g, o}`` (attention; no
+    k and v with ``kv_from``), ``l<i>.mix.{q, k, v, g, o, norm, i, i.b, f, f.b}`` (mlstm), ``l<i>.mix.{q, k, v, g, o, norm,
+    a1, a2, a2.b}`` (gla, whose low rank is the shape of ``a1``); ``l<i>.mlp.{gate, up, down}`` or ``l<i>.mlp.{router,
+    correction, e<k>.{gate, up, down}}``; ``final.norm``.  Linear weights are [out, in]; the input projections of a
+    mixer are fused row-wise here.  Every tensor the model holds must be found, and every tensor of the file must
+    have a place."""
+    from ..engine.config import GatedLinearSpec, MatrixMemorySpec, NormedAttentionSpec
+
+    pat = re.compile(r"l(\d+)\.(.+)")
+    expert = re.compile(r"mlp\.e(\d+)\.(gate|up|down)")
+    seen: set[str] = set()
+
+    def put(dst: torch.Tensor, src: torch.Tensor, what: str) -> None:
+        if tuple(dst.shape) != tuple(src.shape):
+            raise ValueError(f"{what}: checkpoint shape {tuple(src.shape)}, model expects {tuple(dst.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+    tensors = list(_iter_safetensors(ckpt_dir))
+    for name, t in tensors:  # the decays' low rank first: it sizes the fused input projection
+        mt = pat.match(name)
+        if mt and mt.group(2) == "mix.a1" and int(mt.group(1)) < len(model.layers):
+            lw = model.layers[int(mt.group(1))]
+            if isinstance(lw.spec.mixer, GatedLinearSpec) and t.dim() == 2 and lw.w_a2.shape[1] != t.shape[0]:
+                model.set_decay_rank(lw, t.shape[0])
+    for name, t in tensors:
+        seen.add(name)
+        if name == "embed":
+            put(model.embed, t, name)
+            continue
+        if name == "final.norm":
+            put(model.norm, t, name)
+            continue
+        mt = pat.match(name)
+        if not mt or int(mt.group(1)) >= len(model.layers):
+            raise ValueError(f"unexpected tensor {name!r}")
+        lw = model.layers[int(mt.group(1))]
+        sub = mt.group(2)
+        m, f = lw.spec.mixer, lw.spec.mlp
+        me = expert.fullmatch(sub)
+        hd, hv = m.heads * m.dim, m.heads * m.vdim
+        rows: dict[str, tuple] = {}
+        if isinstance(m, NormedAttentionSpec):
+            kd, kv = m.kv_heads * m.dim, m.kv_heads * m.vdim
+            if m.kv_from is None:
+                rows = {"mix.q": (0, hd), "mix.k": (hd, hd + kd), "mix.v": (hd + kd, hd + kd + kv),
+                        "mix.g": (hd + kd + kv, hd + kd + kv + hv)}
+            else:
+                rows = {"mix.q": (0, hd), "mix.g": (hd, hd + hv)}
+        else:
+            rows = {"mix.q": (0, hd), "mix.k": (hd, 2 * hd), "mix.v": (2 * hd, 2 * hd + hv),
+                    "mix.g": (2 * hd + hv, 2 * hd + 2 * hv)}
+            if isinstance(m, GatedLinearSpec):
+                rows["mix.a1"] = (2 * hd + 2 * hv, lw.w_in.shape[0])
+        if sub == "norm1":
+            put(lw.norm1, t, name)
+        elif sub == "norm2" and f is not None:
+            put(lw.norm2, t, name)
+        elif sub in rows:
+            a, b = rows[sub]
+            put(lw.w_in[a:b], t, name)
+        elif sub == "mix.o":
+            put(lw.w_o, t, name)
+        elif sub == "mix.sink" and isinstance(m, NormedAttentionSpec):
+            put(lw.sink, t, name)
+        elif sub == "mix.norm" and not isinstance(m, NormedAttentionSpec):
+            put(lw.h_norm, t, name)
+        elif sub == "mix.i" and isinstance(m, MatrixMemorySpec):
+            put(lw.w_if[:m.heads], t, name)
+        elif sub == "mix.f" and isinstance(m, MatrixMemorySpec):
+            put(lw.w_if[m.heads:], t, name)
+        elif sub == "mix.i.b" and isinstance(m, MatrixMemorySpec):
+            put(lw.b_i, t, name)
+        elif sub == "mix.f.b" and isinstance(m, MatrixMemorySpec):
+            put(lw.b_f, t, name)
+        elif sub == "mix.a2" and isinstance(m, GatedLinearSpec):
+            put(lw.w_a2, t, name)
+        elif sub == "mix.a2.b" and isinstance(m, GatedLinearSpec):
+            put(lw.a2_b, t, name)
+        elif sub == "mlp.gate" and f is not None and f.kind == "dense":
+            put(lw.w_gu[:f.ff], t, name)
+        elif sub == "mlp.up" and f is not None and f.kind == "dense":
+            put(lw.w_gu[f.ff:], t, name)
+        elif sub == "mlp.down" and f is not None and f.kind == "dense":
+            put(lw.w_down, t, name)
+        elif sub == "mlp.router" and f is not None and f.kind == "moe":
+            put(lw.router, t, name)
+        elif sub == "mlp.correction" and f is not None and f.kind == "moe":
+            put(lw.correction, t, name)
+        elif me and f is not None and f.kind == "moe" and int(me.group(1)) < f.experts:
+            e, which = int(me.group(1)), me.group(2)
+            if which == "gate":
+                put(lw.w13[e, :f.ff], t, name)
+            elif which == "up":
+                put(lw.w13[e, f.ff:], t, name)
+            else:
+                put(lw.w2[e], t, name)
+        else:
+            raise ValueError(f"unexpected tensor {name!r}")
+    want = {"embed", "final.norm"}
+    for i, lw in enumerate(model.layers):
+        m, f = lw.spec.mixer, lw.spec.mlp
+        want |= {f"l{i}.norm1", f"l{i}.mix.q", f"l{i}.mix.g", f"l{i}.mix.o"}
+        if isinstance(m, NormedAttentionSpec):
+            want.add(f"l{i}.mix.sink")
+            if m.kv_from is None:
+                want |= {f"l{i}.mix.k", f"l{i}.mix.v"}
+        else:
+            want |= {f"l{i}.mix.k", f"l{i}.mix.v", f"l{i}.mix.norm"}
+            want |= ({f"l{i}.mix.{k}" for k in ("i", "i.b", "f", "f.b")} if isinstance(m, MatrixMemorySpec)
+                     else {f"l{i}.mix.{k}" for k in ("a1", "a2", "a2.b")})
+        if f is not None:
+            want.add(f"l{i}.norm2")
+            if f.kind == "dense":
+                want |= {f"l{i}.mlp.{k}" for k in ("gate", "up", "down")}
+            else:
+                want |= {f"l{i}.mlp.router", f"l{i}.mlp.correction"}
+                want |= {f"l{i}.mlp.e{e}.{k}" for e in range(f.experts) for k in ("gate", "up", "down")}
     if want - seen:
         raise ValueError(f"checkpoint lacks {sorted(want - seen)[:8]}")

@@ -731,6 +731,9 @@ TILE_CUS = 256
 _tile_enabled = os.environ.get("VPSA_TILE_GEMM", "1") != "0"
 
 
+TILE_GELU_GLU = False  # the gated gelu unit in the prefill GEMM's epilogue (tile_gemm(gelu_mul=True))
+
+
 def set_tile_gemm(on: bool) -> bool:
     """Switch the hand-written prefill GEMM on or off (A/B timing); returns the old value."""
     global _tile_enabled
@@ -1119,7 +1122,7 @@ def moe_mfma_supported(hidden: int, inter: int) -> bool:
     return hidden % 128 == 0 and inter % 512 == 0
 
 
-def moe_experts_grouped(x, w13, w2, ids, weights, foreign=False):
+def moe_experts_grouped(x, w13, w2, ids, weights, foreign=False, combine=True):
     """Expert MLP for a decode-sized batch: out[t] = sum_k weights[t,k] * MLP_{ids[t,k]}(x[t]).
     ``foreign``: ids may equal the expert count (a pair of an expert held by another rank, weight
     0): those pairs sort behind the last expert and no kernel touches them.
@@ -1143,6 +1146,8 @@ def moe_experts_grouped(x, w13, w2, ids, weights, foreign=False):
                                   _p(act), _p(y), c_int(t), c_int(k), c_int(n_experts),
                                   c_int(hidden), c_int(inter), _stream())
     _check(rc, "moe_mfma")
+    if not combine:  # the caller sums the pairs itself (y in sorted order, pos: the sorted row of pair t * K + k)
+        return y, pos
     return moe_combine(y, weights, pos, t)
 
 
@@ -1237,7 +1242,7 @@ def grouped_gemm_supported(n: int, k: int, silu_mul: bool = False) -> bool:
     return k % 64 == 0 and (not silu_mul or (n // 2) % 32 == 0)
 
 
-def moe_experts_prefill(x, w13, w2, ids, weights, gather=True, foreign=False):
+def moe_experts_prefill(x, w13, w2, ids, weights, gather=True, foreign=False, combine=True):
     """Expert MLP for prefill-sized batches: the (token, k) pairs are sorted by expert on the device
     and two grouped matrix-core GEMMs run over all experts at once: gate_up gathers its token
     rows by index and fuses silu(gate) * up, down writes the sorted rows that the weighted combine
@@ -1256,6 +1261,8 @@ def moe_experts_prefill(x, w13, w2, ids, weights, gather=True, foreign=False):
     else:  # copy the rows into sorted order first (timing comparison)
         act = gg(moe_permute(x, sorted_tok), w13, offsets, rows=t * k, silu_mul=True)
     y = gg(act, w2, offsets, rows=t * k)
+    if not combine:  # the caller sums the pairs itself
+        return y, pos
     return moe_combine(y, weights, pos, t)
 
 
@@ -1328,9 +1335,11 @@ def lora_expand(h, bs, slots, y, r_pad):
 
 # --------------------------------------------------------------------------- latent attention, group routing, fp32 residual
 from .latent import (add_rms_norm, build_latent_tiles, embed_scale, gate_up_glu_clamp, gather_rows, glu_clamp,  # noqa: E402,F401
+                     gate_up_act, glu_act, rms_norm_add, route_softmax,
                      group_topk, latent_attention, moe_glu_grouped, moe_glu_grouped_supported, up_relu_sq,
                      latent_kv_write, latent_mfma_supported, latent_tile_kernel_takes, moe_finish, relu_sq, rms_norm_rows, rope_pairs, sigmoid_gate)
 
 # --------------------------------------------------------------------------- recurrent mixers, windowed attention, Dynamic Tanh
 from .seqmix import (add_dyt_norm, build_scan_pieces, build_window_tiles, head_rms_norm, mix_heads, recurrent_scan, short_conv_qkv,  # noqa: E402,F401
+                     gla_prepare, head_finish, mlstm_prepare, prepared_scan, qk_norm_write, scan_state_cols,
                      up_xielu, window_attention, window_cache_elems, window_decode_splits, window_mfma_supported, xielu)

@@ -78,6 +78,23 @@ def add_rms_norm(residual, delta, weight, eps: float, out_dtype, want_out: bool 
     return y
 
 
+def rms_norm_add(residual, delta, weight, eps: float, out_dtype, want_out: bool = True):
+    """A norm on a sublayer's output: residual (fp32, in place) += rmsnorm(delta) * weight.  ``delta`` is in
+    ``out_dtype`` or fp32 (a mixture's sum).  Returns the new residual rounded to ``out_dtype``: the next
+    sublayer's input, for designs whose sublayers read the stream itself."""
+    if not residual.is_cuda:
+        return reference.rms_norm_add(residual, delta, weight, eps, out_dtype, want_out)
+    o = _ops()
+    _f32(residual, weight)
+    t, n = residual.shape
+    assert _rows(delta) and delta.shape == residual.shape and delta.dtype in (out_dtype, torch.float32)
+    y = torch.empty((t, n), dtype=out_dtype, device=residual.device) if want_out else None
+    o._check(o._kernels().vpsa_rmsnorm_add(o._p(residual), o._p(delta), c_long(delta.stride(0)),
+                                           c_int(1 if delta.dtype == torch.float32 else 0), o._p(weight), o._p(y), c_int(t),
+                                           c_int(n), c_float(eps), c_int(_DT[out_dtype]), o._stream()), "rms_norm_add")
+    return y
+
+
 def rms_norm_rows(x, weight, eps: float):
     """rmsnorm over the columns of a 2-D view (a column range of a wider projection output)."""
     if not x.is_cuda:
@@ -259,6 +276,59 @@ def glu_clamp(x, limit: float, alpha: float = 1.702, up_bias: float = 1.0):
                                          c_float(limit), c_float(alpha), c_float(up_bias), c_int(_dt(x)), o._stream()),
              "glu_clamp")
     return y
+
+
+GLU_ACTS = {"silu": 0, "gelu_tanh": 1}
+
+
+def glu_act(x, act: str):
+    """x [rows, 2 I] = gate | up  ->  act(gate) * up, act = silu or the tanh form of gelu."""
+    if not x.is_cuda:
+        return reference.glu_act(x, act)
+    o = _ops()
+    assert _rows(x) and x.shape[1] % 2 == 0
+    inter = x.shape[1] // 2
+    y = torch.empty((x.shape[0], inter), dtype=x.dtype, device=x.device)
+    o._check(o._kernels().vpsa_glu_act(o._p(x), c_long(x.stride(0)), o._p(y), c_int(x.shape[0]), c_int(inter),
+                                       c_int(GLU_ACTS[act]), c_int(_dt(x)), o._stream()), "glu_act")
+    return y
+
+
+def gate_up_act(x, w_gate_up, act: str, packed=None):
+    """act(x @ Wg.T) * (x @ Wu.T) for ``w_gate_up = [Wg; Wu]``.  silu in bf16 is the fused path of the other
+    decoders (``gate_up_silu``); the tanh form of gelu runs in the prefill GEMM's epilogue when that kernel
+    takes the shape; everything else is the projection and the activation kernel."""
+    o = _ops()
+    if act == "silu" and x.is_cuda and x.dtype == torch.bfloat16:
+        return o.gate_up_silu(x, w_gate_up, packed)
+    rows = o.tile_rows(x, w_gate_up, True) if (x.is_cuda and act == "gelu_tanh" and o.TILE_GELU_GLU) else 0
+    if rows == x.shape[0] and rows:
+        return o.tile_gemm(x, w_gate_up, gelu_mul=True)
+    return glu_act(o.linear(x, w_gate_up), act)
+
+
+def route_softmax(logits, n: int, experts: int, groups: int, keep: int, topk: int, bias=None, route_scale: float = 1.0,
+                  park_in_bucket: bool = True):
+    """Router logits fp32 [T, >= n] -> (weights fp32 [T, topk], ids int32 [T, topk], gate fp32 [T] or None).
+    Scores are the softmax over all ``n`` outputs; an output is chosen by score + ``bias`` (fp32 [n]) and
+    weighted by the score alone (times ``route_scale``, not renormalised).  Outputs form ``groups`` equal
+    runs of neighbours, a group scores its largest biased score, and only outputs of the ``keep`` best
+    groups can be chosen.  Outputs ``experts .. n`` are identity experts (their output is the token itself):
+    a chosen one leaves the pair list (weight 0, id ``experts`` with ``park_in_bucket``, a bucket that sorting
+    kernels put behind the last expert and no product visits, else id 0) and its score is added to ``gate``."""
+    if not logits.is_cuda:
+        return reference.route_softmax(logits, n, experts, groups, keep, topk, bias, route_scale, park_in_bucket)
+    o = _ops()
+    _f32(logits, bias)
+    t = logits.shape[0]
+    w = torch.empty((t, topk), dtype=torch.float32, device=logits.device)
+    ids = torch.empty((t, topk), dtype=torch.int32, device=logits.device)
+    gate = torch.empty((t,), dtype=torch.float32, device=logits.device) if experts < n else None
+    o._check(o._kernels().vpsa_route_softmax(o._p(logits), c_int(logits.shape[1]), o._p(bias), o._p(w), o._p(ids),
+                                             o._p(gate), c_int(t), c_int(n), c_int(experts), c_int(groups), c_int(keep),
+                                             c_int(topk), c_float(route_scale), c_int(experts if park_in_bucket else 0),
+                                             o._stream()), "route_softmax")
+    return w, ids, gate
 
 
 def group_topk(logits, experts: int, groups: int, keep: int, topk: int, route_scale: float, extra: bool = False):

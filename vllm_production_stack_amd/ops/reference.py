@@ -14,6 +14,8 @@ contiguous KiB; head sizes that are not a multiple of 32 use one block of the wh
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 PAGE = 64
@@ -358,6 +360,39 @@ def add_rms_norm(residual, delta, weight, eps, out_dtype, want_out=True):
     return (residual * inv * weight).to(out_dtype)
 
 
+def rms_norm_add(residual, delta, weight, eps, out_dtype, want_out=True):
+    d = delta.float()
+    residual.add_(d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * weight)
+    return residual.to(out_dtype) if want_out else None
+
+
+def glu_act(x, act):
+    inter = x.shape[1] // 2
+    g, u = x[:, :inter].float(), x[:, inter:].float()
+    a = torch.nn.functional.silu(g) if act == "silu" else torch.nn.functional.gelu(g, approximate="tanh")
+    return (a * u).to(x.dtype)
+
+
+def route_softmax(logits, n, experts, groups, keep, topk, bias, route_scale, park_in_bucket):
+    t = logits.shape[0]
+    s = torch.softmax(logits[:, :n].float(), dim=-1)
+    c = s + bias if bias is not None else s.clone()
+    per = n // groups
+    score = c.view(t, groups, per).max(-1).values
+    order = torch.sort(score, dim=-1, descending=True, stable=True).indices[:, :keep]
+    allowed = torch.zeros((t, groups), dtype=torch.bool)
+    allowed.scatter_(1, order, True)
+    c = torch.where(allowed[:, :, None].expand(t, groups, per).reshape(t, n), c, torch.full_like(c, -math.inf))
+    ids = torch.sort(c, dim=-1, descending=True, stable=True).indices[:, :topk]
+    w = s.gather(1, ids) * route_scale
+    if experts == n:
+        return w, ids.int(), None
+    ident = ids >= experts
+    gate = torch.where(ident, w, torch.zeros_like(w)).sum(-1)
+    ids = torch.where(ident, torch.full_like(ids, experts if park_in_bucket else 0), ids)
+    return torch.where(ident, torch.zeros_like(w), w), ids.int(), gate
+
+
 def rms_norm_rows(x, weight, eps):
     xf = x.float()
     return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * weight).to(x.dtype)
@@ -522,6 +557,101 @@ def recurrent_scan(proj, q_col, k_col, v_col, heads, dim, vdim, gated, state, st
     return out
 
 
+def gla_prepare(proj, q_col, k_col, z, z_bias, heads, dim, q_scale, tau):
+    t = proj.shape[0]
+    q = proj[:, q_col:q_col + heads * dim].float() * q_scale
+    k = proj[:, k_col:k_col + heads * dim].float()
+    a = torch.exp(torch.nn.functional.logsigmoid(z.float() + z_bias) / tau)
+    return torch.stack([q.view(t, heads, dim), k.view(t, heads, dim), a.view(t, heads, dim)], dim=2).contiguous()
+
+
+def mlstm_prepare(proj, q_col, k_col, gate_logits, bias_i, bias_f, cap, heads, dim, q_scale, state, m_off, seq_cu,
+                  seq_state, positions):
+    t = proj.shape[0]
+    q = proj[:, q_col:q_col + heads * dim].float().view(t, heads, dim) * q_scale
+    k = proj[:, k_col:k_col + heads * dim].float().view(t, heads, dim)
+    gi = cap * torch.tanh((gate_logits[:, :heads] + bias_i) / cap)
+    gf = torch.nn.functional.logsigmoid(cap * torch.tanh((gate_logits[:, heads:] + bias_f) / cap))
+    dec = torch.zeros((t, heads), dtype=torch.float32)
+    wr = torch.zeros((t, heads), dtype=torch.float32)
+    mrow = torch.zeros((t, heads), dtype=torch.float32)
+    cu, slots = seq_cu.tolist(), seq_state.tolist()
+    for s, slot in enumerate(slots):
+        r0, r1 = cu[s], cu[s + 1]
+        if slot < 0 or r1 <= r0:
+            continue
+        m = state[slot, m_off:m_off + heads]
+        if int(positions[r0]) == 0:
+            m.zero_()
+        for r in range(r0, r1):
+            new = torch.maximum(gf[r] + m, gi[r])
+            dec[r] = torch.exp(gf[r] + m - new)
+            wr[r] = torch.exp(gi[r] - new)
+            mrow[r] = new
+            m.copy_(new)
+    prep = torch.stack([q, k * wr[:, :, None], dec[:, :, None].expand(t, heads, dim)], dim=2).contiguous()
+    return prep, mrow
+
+
+def prepared_scan(prep, proj, v_col, heads, dim, vdim, cols, unit_col, state, state_off, seq_cu, seq_state, positions):
+    t = proj.shape[0]
+    out = torch.zeros((t, heads, cols), dtype=torch.float32)
+    v = torch.zeros((t, heads, cols), dtype=torch.float32)
+    v[:, :, :vdim] = proj[:, v_col:v_col + heads * vdim].float().view(t, heads, vdim)
+    if unit_col:
+        v[:, :, vdim] = 1.0
+    cu, slots = seq_cu.tolist(), seq_state.tolist()
+    for s, slot in enumerate(slots):
+        r0, r1 = cu[s], cu[s + 1]
+        if slot < 0 or r1 <= r0:
+            continue
+        S = state[slot, state_off:state_off + heads * dim * cols].view(heads, dim, cols)
+        if int(positions[r0]) == 0:
+            S.zero_()
+        for r in range(r0, r1):
+            S.mul_(prep[r, :, 2].unsqueeze(-1)).add_(prep[r, :, 1].unsqueeze(-1) * v[r].unsqueeze(1))
+            out[r] = torch.einsum("hdv,hd->hv", S, prep[r, :, 0])
+    return out
+
+
+def head_finish(o, eps, out_dtype, vdim, stab, unit, weight, gate, gate_act):
+    t, heads, _ = o.shape
+    y = o[:, :, :vdim]
+    if stab is not None:
+        y = y / (torch.maximum(o[:, :, vdim].abs(), torch.exp(-stab)) + 1e-6)[:, :, None]
+    if unit:
+        y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps)
+    if weight is not None:
+        y = y * (weight if weight.numel() == vdim else weight.view(heads, vdim))
+    y = y.reshape(t, heads * vdim)
+    if gate is not None:
+        g = gate.float()
+        y = y * (torch.nn.functional.silu(g) if gate_act == "silu" else torch.sigmoid(g))
+    return y.to(out_dtype)
+
+
+def qk_norm_write(proj, heads, kv_heads, dim, vdim, positions, slots, pool, cache_off, eps, temp_coef, temp_every, own):
+    t = proj.shape[0]
+    nq, nk = heads * dim, kv_heads * dim
+
+    def unit(x):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+    q = unit(proj[:, :nq].float().view(t, heads, dim))
+    if temp_coef != 0.0:
+        steps = torch.floor((positions.double() + 1.0) / temp_every).float()
+        q = q * (1.0 + temp_coef * torch.log(steps + 1.0))[:, None, None]
+    if own:
+        k = unit(proj[:, nq:nq + nk].float().view(t, kv_heads, dim)).to(pool.dtype)
+        v = proj[:, nq + nk:nq + nk + kv_heads * vdim].reshape(t, kv_heads, vdim).to(pool.dtype)
+        kc, vc = window_cache_views(pool, cache_off, kv_heads, dim, vdim)
+        ok = slots >= 0
+        pg, off = (slots[ok] // PAGE).long(), (slots[ok] % PAGE).long()
+        kc[pg, off] = k[ok]
+        vc[pg, off] = v[ok]
+    return q.to(proj.dtype)
+
+
 def head_rms_norm(o, eps, weight, gate, out_dtype):
     t, heads, vdim = o.shape
     y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
@@ -579,7 +709,7 @@ def short_conv_qkv(proj, conv_w, heads, kv_heads, dim, vdim, state, state_off, s
 
 
 def window_attention(q, pool, cache_off, kv_heads, vdim, block_tables, row_seq, positions, window, keep_first, scale,
-                     softcap, sink, out):
+                     softcap, sink, out, own_values=False):
     t, heads, dim = q.shape
     kc, vc = window_cache_views(pool, cache_off, kv_heads, dim, vdim)
     rep = heads // kv_heads
@@ -598,7 +728,10 @@ def window_attention(q, pool, cache_off, kv_heads, vdim, block_tables, row_seq, 
         mx = torch.maximum(sc.max(-1).values, sink)
         e = torch.exp(sc - mx[:, None])
         w = e / (e.sum(-1) + torch.exp(sink - mx))[:, None]
-        out[r] = torch.einsum("hk,kgv->hgv", w, vv)
+        if own_values:
+            out[r, :, 0] = torch.einsum("hk,khv->hv", w, vv.repeat_interleave(rep, dim=1))
+        else:
+            out[r] = torch.einsum("hk,kgv->hgv", w, vv)
     return out
 
 

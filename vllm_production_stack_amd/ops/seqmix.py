@@ -176,6 +176,143 @@ def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: in
     return out
 
 
+def gla_prepare(proj, q_col: int, k_col: int, z, z_bias, heads: int, dim: int, q_scale: float, tau: float):
+    """What a gated-linear-attention recurrence takes besides v, fp32 [T, heads, 3, dim]: q * q_scale | k | a with
+    the decay a = sigmoid(z + z_bias)^(1 / tau) per head and key channel.  q and k are column ranges of ``proj``,
+    ``z`` [T, heads * dim] the decay's pre-activation (activation dtype), ``z_bias`` fp32."""
+    if not proj.is_cuda:
+        return reference.gla_prepare(proj, q_col, k_col, z, z_bias, heads, dim, q_scale, tau)
+    o = _ops()
+    _f32(z_bias)
+    t = proj.shape[0]
+    assert _rows(proj) and _rows(z) and z.shape == (t, heads * dim) and max(q_col, k_col) + heads * dim <= proj.shape[1]
+    prep = torch.empty((t, heads, 3, dim), dtype=torch.float32, device=proj.device)
+    o._check(o._kernels().vpsa_gla_prepare(o._p(proj), c_long(proj.stride(0)), c_int(q_col), c_int(k_col), o._p(z),
+                                           c_long(z.stride(0)), o._p(z_bias), c_int(heads), c_int(dim), c_float(q_scale),
+                                           c_float(tau), o._p(prep), c_int(t), c_int(_dt(proj, z)), o._stream()),
+             "gla_prepare")
+    return prep
+
+
+def mlstm_prepare(proj, q_col: int, k_col: int, gate_logits, bias_i, bias_f, cap: float, heads: int, dim: int,
+                  q_scale: float, state, m_off: int, seq_cu, seq_state, positions):
+    """Gates of a matrix memory with exponential gating.  ``gate_logits`` fp32 [T, 2 heads] = input | forget gate
+    pre-activations (biases apart); i = cap tanh((x_i + b_i) / cap), f = logsigmoid(cap tanh((x_f + b_f) / cap)).
+    The running maximum m_t = max(f_t + m_(t-1), i_t) starts at 0 with the sequence and is carried in the
+    sequence's state slot (``heads`` floats at ``m_off``).  Returns (prep fp32 [T, heads, 3, dim] =
+    q * q_scale | k * exp(i_t - m_t) | exp(f_t + m_(t-1) - m_t), m fp32 [T, heads])."""
+    if not proj.is_cuda:
+        return reference.mlstm_prepare(proj, q_col, k_col, gate_logits, bias_i, bias_f, cap, heads, dim, q_scale, state,
+                                       m_off, seq_cu, seq_state, positions)
+    o = _ops()
+    _f32(gate_logits, bias_i, bias_f, state)
+    _i32(seq_cu, seq_state, positions)
+    t = proj.shape[0]
+    assert _rows(proj) and gate_logits.shape == (t, 2 * heads) and max(q_col, k_col) + heads * dim <= proj.shape[1]
+    assert m_off + heads <= state.shape[1] and seq_cu.numel() == seq_state.numel() + 1
+    prep = torch.empty((t, heads, 3, dim), dtype=torch.float32, device=proj.device)
+    ab = torch.empty((t, heads, 2), dtype=torch.float32, device=proj.device)
+    mrow = torch.empty((t, heads), dtype=torch.float32, device=proj.device)
+    o._check(o._kernels().vpsa_mlstm_prepare(
+        o._p(proj), c_long(proj.stride(0)), c_int(q_col), c_int(k_col), o._p(gate_logits), o._p(bias_i), o._p(bias_f),
+        c_float(cap), c_int(heads), c_int(dim), c_float(q_scale), _at(state, m_off), c_long(state.stride(0)), o._p(seq_cu),
+        o._p(seq_state), c_int(seq_state.numel()), o._p(positions), o._p(ab), o._p(mrow), o._p(prep), c_int(t),
+        c_int(_dt(proj)), o._stream()), "mlstm_prepare")
+    return prep, mrow
+
+
+def scan_state_cols(vdim: int, unit_col: bool = False) -> int:
+    """Columns per key channel of a prepared recurrence's state: the values, one more for the normaliser when
+    ``unit_col``, rounded up to whole float4."""
+    return (vdim + 4) // 4 * 4 if unit_col else vdim
+
+
+def prepared_scan(prep, proj, v_col: int, heads: int, dim: int, vdim: int, state, state_off: int, seq_cu, seq_state,
+                  positions, *, unit_col: bool = False, pieces=None):
+    """``recurrent_scan`` over rows a caller prepared: prep fp32 [T, heads, 3, dim] = q' | k' | a (per row, head and
+    key channel), S <- diag(a_t) S + k'_t v_t^T, o_t = S^T q'_t, with S carried in the sequence's state slot.
+    v is a column range of ``proj``.  ``unit_col``: the state gets one more value column that is fed with ones, so
+    that it accumulates n_t = a_t n_(t-1) + k'_t and its read-out is n_t . q'_t (a normaliser); the state then
+    has ``scan_state_cols(vdim, True)`` columns.  Returns o fp32 [T, heads, state columns]."""
+    cols = scan_state_cols(vdim, unit_col)
+    if not proj.is_cuda:
+        return reference.prepared_scan(prep, proj, v_col, heads, dim, vdim, cols, unit_col, state, state_off, seq_cu,
+                                       seq_state, positions)
+    o = _ops()
+    _f32(prep, state)
+    _i32(seq_cu, seq_state, positions)
+    t = proj.shape[0]
+    assert _rows(proj) and v_col + heads * vdim <= proj.shape[1] and prep.shape == (t, heads, 3, dim)
+    assert state_off + heads * dim * cols <= state.shape[1] and seq_cu.numel() == seq_state.numel() + 1
+    out = torch.empty((t, heads, cols), dtype=torch.float32, device=proj.device)
+    pc = sp = ws_state = ws_decay = None
+    n_pieces = 0
+    if pieces is not None:
+        pc, sp = pieces
+        _i32(pc, sp)
+        n_pieces = pc.shape[0]
+        assert pc.shape[1] == 3 and sp.numel() == seq_cu.numel()
+        ws_state = torch.empty((n_pieces, heads, dim, cols), dtype=torch.float32, device=proj.device)
+        ws_decay = torch.empty((n_pieces, heads, dim), dtype=torch.float32, device=proj.device)
+    o._check(o._kernels().vpsa_prepared_scan(
+        o._p(proj), c_long(proj.stride(0)), c_int(v_col), c_int(vdim), c_int(1 if unit_col else 0), c_int(heads),
+        c_int(dim), c_int(cols), o._p(prep), _at(state, state_off), c_long(state.stride(0)), o._p(seq_cu),
+        o._p(seq_state), c_int(seq_state.numel()), o._p(positions), o._p(out), o._p(pc), o._p(sp), c_int(n_pieces),
+        o._p(ws_state), o._p(ws_decay), c_int(t), c_int(_dt(proj)), o._stream()), "prepared_scan")
+    return out
+
+
+GATE_ACTS = {"silu": 0, "sigmoid": 1}
+
+
+def head_finish(o_heads, eps: float, out_dtype, *, vdim: int | None = None, stab=None, unit: bool = True, weight=None,
+                gate=None, gate_act: str = "silu"):
+    """Head outputs o fp32 [T, heads, cols] (the first ``vdim`` columns count) -> [T, heads * vdim] in ``out_dtype``.
+    In this order, each part optional: ``stab`` (fp32 [T, heads], the gates' running maximum m): column ``vdim`` of o
+    is a normaliser's read-out n . q and the output is divided by max(|n . q|, exp(-m)) + 1e-6; ``unit``: every head
+    divided by its root mean square (eps inside the root); ``weight`` fp32 [vdim] (shared by the heads) or
+    [heads * vdim]; ``gate`` (a [T, heads * vdim] view of a wider projection) through silu or sigmoid."""
+    t, heads, cols = o_heads.shape
+    vdim = cols if vdim is None else vdim
+    if not o_heads.is_cuda:
+        return reference.head_finish(o_heads, eps, out_dtype, vdim, stab, unit, weight, gate, gate_act)
+    o = _ops()
+    _f32(o_heads, weight, stab)
+    assert gate is None or (_rows(gate) and gate.shape == (t, heads * vdim) and gate.dtype == out_dtype)
+    assert weight is None or weight.numel() in (vdim, heads * vdim)
+    assert stab is None or (stab.shape == (t, heads) and cols > vdim)
+    y = torch.empty((t, heads * vdim), dtype=out_dtype, device=o_heads.device)
+    o._check(o._kernels().vpsa_head_finish(
+        o._p(o_heads), c_int(cols), o._p(stab), c_int(1 if unit else 0), o._p(weight),
+        c_int(1 if (weight is not None and weight.numel() != vdim) else 0), o._p(gate),
+        c_long(gate.stride(0) if gate is not None else 0), c_int(GATE_ACTS[gate_act]), o._p(y), c_int(t), c_int(heads),
+        c_int(vdim), c_float(eps), c_int(_DT[out_dtype]), o._stream()), "head_finish")
+    return y
+
+
+def qk_norm_write(proj, heads: int, kv_heads: int, dim: int, vdim: int, positions, slots, pool, cache_off: int,
+                  eps: float, temp_coef: float = 0.0, temp_every: float = 1.0, own: bool = True):
+    """Rows of a fused projection, q | k | v (``own``) or q alone (a layer that reads another layer's cache
+    entries): every q and k head is divided by its root mean square (eps inside the root, no weight); q at
+    position p is then multiplied by 1 + temp_coef ln(floor((p + 1) / temp_every) + 1).  k and v go to the paged
+    cache at ``slots`` (< 0: not cached) in the layout ``window_attention`` reads; returns q [T, heads, dim]."""
+    if not proj.is_cuda:
+        return reference.qk_norm_write(proj, heads, kv_heads, dim, vdim, positions, slots, pool, cache_off, eps,
+                                       temp_coef, temp_every, own)
+    o = _ops()
+    _i32(positions)
+    t = proj.shape[0]
+    chans = heads * dim + (kv_heads * (dim + vdim) if own else 0)
+    assert _rows(proj) and proj.shape[1] >= chans and slots.dtype == torch.int64
+    assert pool.dim() == 2 and pool.stride(1) == 1 and cache_off + window_cache_elems(kv_heads, dim, vdim) <= pool.shape[1]
+    q = torch.empty((t, heads, dim), dtype=proj.dtype, device=proj.device)
+    o._check(o._kernels().vpsa_qk_norm_write(
+        o._p(proj), c_long(proj.stride(0)), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim), c_int(1 if own else 0),
+        o._p(positions), o._p(slots), c_float(eps), c_float(temp_coef), c_float(temp_every), o._p(q), _at(pool, cache_off),
+        c_long(pool.stride(0)), c_int(t), c_int(_dt(proj, pool)), o._stream()), "qk_norm_write")
+    return q
+
+
 def head_rms_norm(o_heads, eps: float, out_dtype, weight=None, gate=None):
     """o fp32 [T, heads, vdim] -> [T, heads * vdim] in ``out_dtype``: every head divided by its root mean
     square (eps inside the root), times ``weight`` (fp32 [vdim], shared by the heads) and times
@@ -236,8 +373,9 @@ def window_tile_slots() -> int:
 WINDOW_MFMA = True      # False: every call takes the plain kernel (A/B runs, tests of the plain kernel)
 
 
-def window_mfma_supported(heads: int, kv_heads: int, dim: int, vdim: int) -> bool:
-    return bool(_ops()._kernels().vpsa_window_mfma_supported(c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim)))
+def window_mfma_supported(heads: int, kv_heads: int, dim: int, vdim: int, own_values: bool = False) -> bool:
+    return bool(_ops()._kernels().vpsa_window_mfma_supported(c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim),
+                                                             c_int(1 if own_values else 0)))
 
 
 def build_window_tiles(q_lens, ctx_lens, heads: int, kv_heads: int):
@@ -268,23 +406,27 @@ def window_decode_splits(rows: int, kv_heads: int, window: int, keep_first: int,
 
 
 def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_tables, row_seq, positions, window: int,
-                     keep_first: int, scale: float, softcap: float, sink, out=None, tiles=None, splits: int = 1):
+                     keep_first: int, scale: float, softcap: float, sink, out=None, tiles=None, splits: int = 1,
+                     own_values: bool = False):
     """Query rows q [T, heads, dim] over their sequences' cached keys: row i at position p sees key j when
     j <= p and (p - j < window or j < keep_first).  score = cap * tanh(q . k * scale / cap) (cap 0: none);
     softmax with ``sink`` [heads] (fp32) in the denominator.  Returns u fp32 [T, heads, kv_heads, vdim]:
-    each head's weights applied to the values of every KV head (``mix_heads`` picks and mixes).
+    each head's weights applied to the values of every KV head (``mix_heads`` picks and mixes).  With
+    ``own_values`` only those of the head's own KV head: u fp32 [T, heads, 1, vdim], the attention output of designs
+    without head mixing (a window of at least the context length makes it plain causal attention).
 
     bf16 rows of a shape the matrix-core kernel tiles take it: decode batches (``row_seq`` None) as they
     are (with ``splits`` key ranges per row, merged by a second launch), prefill rows when ``tiles`` (the
     device copy of ``build_window_tiles``) describes them.  Everything else takes the plain kernel."""
     t, heads, dim = q.shape
+    vsets = 1 if own_values else kv_heads
     if out is None:
-        out = torch.empty((t, heads, kv_heads, vdim), dtype=torch.float32, device=q.device)
+        out = torch.empty((t, heads, vsets, vdim), dtype=torch.float32, device=q.device)
     if t == 0:
         return out
     if not q.is_cuda:
         return reference.window_attention(q, pool, cache_off, kv_heads, vdim, block_tables, row_seq, positions, window,
-                                          keep_first, scale, softcap, sink, out)
+                                          keep_first, scale, softcap, sink, out, own_values)
     o = _ops()
     _f32(sink, out)
     _i32(row_seq, positions)
@@ -293,7 +435,9 @@ def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_ta
     esz = pool.element_size()
     assert (cache_off * esz) % 16 == 0 and (pool.stride(0) * esz) % 16 == 0 and pool.data_ptr() % 16 == 0
     dt = _dt(q, pool)
-    if (WINDOW_MFMA and dt == 0 and (tiles is not None or row_seq is None) and window_mfma_supported(heads, kv_heads, dim, vdim)
+    own = c_int(1 if own_values else 0)
+    if (WINDOW_MFMA and dt == 0 and (tiles is not None or row_seq is None)
+            and window_mfma_supported(heads, kv_heads, dim, vdim, own_values)
             and q.data_ptr() % 16 == 0 and out.data_ptr() % 16 == 0):
         ws_o = ws_ml = None
         if tiles is not None:
@@ -301,20 +445,20 @@ def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_ta
             splits = 1
         elif splits > 1:
             assert out.is_contiguous()
-            ws_o = torch.empty((t * heads * splits * kv_heads * vdim,), dtype=torch.float32, device=q.device)
+            ws_o = torch.empty((t * heads * splits * vsets * vdim,), dtype=torch.float32, device=q.device)
             ws_ml = torch.empty((t * heads * splits * 2,), dtype=torch.float32, device=q.device)
         o._check(o._kernels().vpsa_window_attention_mfma(
             o._p(q), c_long(q.stride(0)), _at(pool, cache_off), c_long(pool.stride(0)), o._p(block_tables),
             c_int(block_tables.stride(0)), o._p(tiles), o._p(positions), o._p(sink), o._p(out),
             c_int(tiles.shape[0] if tiles is not None else t), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim),
             c_int(window), c_int(keep_first), c_float(scale), c_float(softcap), c_int(splits), o._p(ws_o), o._p(ws_ml),
-            o._stream()), "window_attention_mfma")
+            own, o._stream()), "window_attention_mfma")
         return out
     o._check(o._kernels().vpsa_window_attention(
         o._p(q), c_long(q.stride(0)), _at(pool, cache_off), c_long(pool.stride(0)), o._p(block_tables),
         c_int(block_tables.stride(0)), o._p(row_seq), o._p(positions), o._p(sink), o._p(out), c_int(t), c_int(heads),
         c_int(kv_heads), c_int(dim), c_int(vdim), c_int(window), c_int(keep_first), c_float(scale), c_float(softcap),
-        c_int(dt), o._stream()), "window_attention")
+        own, c_int(dt), o._stream()), "window_attention")
     return out
 
 
