@@ -1,6 +1,6 @@
 """Prefill and decode throughput of one decoder design beside the closest existing one at equal size.
 
-    python bench.py --arch-compare zururax|revelix [--arch-sizes s,m] [--arch-prompt 4096] [--arch-batch 32]
+    python bench.py --arch-compare zururax|revelix|pelatar [--arch-sizes s,m] [--arch-prompt 4096] [--arch-batch 32]
 
 Random weights at layer shapes of real models (a few layers each); both models run through the same
 engine (scheduler, paged pool, HIP-graph decode).  Prefill: prompts of --arch-prompt tokens in chunks of
@@ -30,6 +30,8 @@ def _configs(design: str, size: str):
     z = SIZES[size]
     if design == "revelix":
         return _revelix_configs(size)
+    if design == "pelatar":
+        return _pelatar_configs(size)
     if design != "zururax":
         raise SystemExit(f"--arch-compare: unknown design {design!r}")
 
@@ -83,6 +85,23 @@ def _revelix_configs(size: str):
                       intermediate_size=(2 * ff // 3 + 255) // 256 * 256, num_layers=4, num_heads=heads,
                       num_kv_heads=heads // 4, head_dim=128, max_position_embeddings=32768)
     return new, old
+
+
+def _pelatar_configs(size: str):
+    """Pelatar (matrix memory | gated linear attention | attention | attention on its neighbour's keys and values;
+    dense gated gelu units and routed silu units with identity experts in turn) beside the closest existing design,
+    Revelix at the same width, depth and head shapes: its recurrences run the same scan kernel, its attention the
+    same tile kernel (there with a window and head mixing), its feed-forward holds the parameters of the dense
+    gated unit here."""
+    from vllm_production_stack_amd.engine.config import pelatar_config, pelatar_stack
+
+    z = SIZES[size]
+    w = z["width"]
+    ff = (8 * w // 3 + 255) // 256 * 256
+    new = pelatar_config(f"pelatar-{size}", VOCAB, w,
+                         pelatar_stack(w, z["heads"], ff, z["experts"] - 4, z["ff"], z["top"], 4),
+                         max_position_embeddings=32768)
+    return new, _revelix_configs(size)[0]
 
 
 def _measure(cfg, a) -> dict:

@@ -40,40 +40,53 @@ def attention_keys_values(w, pre, h, m, eps):
     return unit_rms(k, eps), v
 
 
-def attention(w, pre, h, m, eps, kv):
-    """Softmax attention of h [T, width] over keys / values ``kv`` (its own, or another layer's)."""
-    t = h.shape[0]
-    hq, g, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = unit_rms((h @ w[pre + "q"].T).view(t, hq, d), eps)
-    temp = m.get("q_temp")
-    if temp:
-        p = torch.arange(t, dtype=F64)
-        q = q * (1.0 + temp["coef"] * torch.log(torch.floor((p + 1) / temp["every"]) + 1.0))[:, None, None]
-    k, v = kv
-    out = torch.zeros(t, hq, dv, dtype=F64)
-    sink = w[pre + "sink"]
-    rep = hq // g
+def temperature(positions, temp):
+    """1 + coef ln(floor((p + 1) / every) + 1), or 1 without a temperature."""
+    p = torch.as_tensor(positions, dtype=F64)
+    if not temp:
+        return torch.ones_like(p)
+    return 1.0 + temp["coef"] * torch.log(torch.floor((p + 1) / temp["every"]) + 1.0)
+
+
+def sink_softmax_attention(q, k, v, pos_q, pos_k, rep, scale, sink):
+    """q [Tq, H, d] at positions pos_q over k [Tk, G, d], v [Tk, G, dv] at pos_k (causal); the sink is one
+    more term exp(sink_h) of every denominator, with no value.  -> [Tq, H, dv]"""
+    tq, hq, _ = q.shape
+    out = torch.zeros(tq, hq, v.shape[2], dtype=F64)
+    hidden = torch.as_tensor(pos_k)[None, :] > torch.as_tensor(pos_q)[:, None]
     for a in range(hq):
-        s = (q[:, a] @ k[:, a // rep].T) * m["scale"]                       # [T, T]
-        s = s.masked_fill(torch.ones(t, t).triu(1).bool(), -math.inf)
+        s = (q[:, a] @ k[:, a // rep].T) * scale
+        s = s.masked_fill(hidden, -math.inf)
         big = torch.maximum(s.max(-1).values, sink[a])
         e = torch.exp(s - big[:, None])
         den = e.sum(-1) + torch.exp(sink[a] - big)
         out[:, a] = (e / den[:, None]) @ v[:, a // rep]
+    return out
+
+
+def attention(w, pre, h, m, eps, kv):
+    """Softmax attention of h [T, width] over keys / values ``kv`` (its own, or another layer's)."""
+    t = h.shape[0]
+    hq, g, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    q = unit_rms((h @ w[pre + "q"].T).view(t, hq, d), eps) * temperature(range(t), m.get("q_temp"))[:, None, None]
+    k, v = kv
+    out = sink_softmax_attention(q, k, v, range(t), range(t), hq // g, m["scale"], w[pre + "sink"])
     gate = torch.sigmoid(h @ w[pre + "g"].T)
     return (out.reshape(t, hq * dv) * gate) @ w[pre + "o"].T
 
 
-def mlstm(w, pre, h, m, eps):
-    """Matrix memory with exponential gates and a running maximum that starts at zero."""
-    t = h.shape[0]
-    nh, d, dv, cap = m["heads"], m["dim"], m["vdim"], m["gate_cap"]
-    q = (h @ w[pre + "q"].T).view(t, nh, d) * d ** -0.5
-    k = (h @ w[pre + "k"].T).view(t, nh, d)
-    v = (h @ w[pre + "v"].T).view(t, nh, dv)
-    gi = cap * torch.tanh((h @ w[pre + "i"].T + w[pre + "i.b"]) / cap)
-    gf = log_sigmoid(cap * torch.tanh((h @ w[pre + "f"].T + w[pre + "f.b"]) / cap))
+def capped_gates(xi, xf, cap):
+    """Log input gate and log forget gate from their pre-activations."""
+    return cap * torch.tanh(xi / cap), log_sigmoid(cap * torch.tanh(xf / cap))
+
+
+def matrix_memory(q, k, v, gi, gf):
+    """q, k [T, H, d] (q already scaled), v [T, H, dv], log gates [T, H] -> ([T, H, dv], the running maxima [T, H]).
+    The maximum starts at zero."""
+    t, nh, d = q.shape
+    dv = v.shape[2]
     out = torch.zeros(t, nh, dv, dtype=F64)
+    tops = torch.zeros(t, nh, dtype=F64)
     for a in range(nh):
         mem = torch.zeros(d, dv, dtype=F64)
         nrm = torch.zeros(d, dtype=F64)
@@ -84,9 +97,38 @@ def mlstm(w, pre, h, m, eps):
             mem = keep * mem + put * torch.outer(k[s, a], v[s, a])
             nrm = keep * nrm + put * k[s, a]
             top = new
+            tops[s, a] = top
             out[s, a] = (mem.T @ q[s, a]) / (max(abs(float(nrm @ q[s, a])), math.exp(-top)) + 1e-6)
+    return out, tops
+
+
+def mlstm(w, pre, h, m, eps):
+    """Matrix memory with exponential gates and a running maximum that starts at zero."""
+    t = h.shape[0]
+    nh, d, dv, cap = m["heads"], m["dim"], m["vdim"], m["gate_cap"]
+    q = (h @ w[pre + "q"].T).view(t, nh, d) * d ** -0.5
+    k = (h @ w[pre + "k"].T).view(t, nh, d)
+    v = (h @ w[pre + "v"].T).view(t, nh, dv)
+    gi, gf = capped_gates(h @ w[pre + "i"].T + w[pre + "i.b"], h @ w[pre + "f"].T + w[pre + "f.b"], cap)
+    out, _ = matrix_memory(q, k, v, gi, gf)
     y = unit_rms(out, eps).reshape(t, nh * dv) * w[pre + "norm"] * torch.sigmoid(h @ w[pre + "g"].T)
     return y @ w[pre + "o"].T
+
+
+def decayed_memory(q, k, v, alpha):
+    """S <- diag(alpha_t) S + k_t v_t^T, o_t = S^T q_t per head; alpha [T, H, d] acts on the rows of key channels."""
+    t, nh, d = q.shape
+    out = torch.zeros(t, nh, v.shape[2], dtype=F64)
+    for a in range(nh):
+        mem = torch.zeros(d, v.shape[2], dtype=F64)
+        for s in range(t):
+            mem = alpha[s, a][:, None] * mem + torch.outer(k[s, a], v[s, a])
+            out[s, a] = mem.T @ q[s, a]
+    return out
+
+
+def channel_decay(z, tau):
+    return torch.exp(log_sigmoid(z) / tau)
 
 
 def gla(w, pre, h, m, eps):
@@ -97,13 +139,7 @@ def gla(w, pre, h, m, eps):
     k = (h @ w[pre + "k"].T).view(t, nh, d)
     v = (h @ w[pre + "v"].T).view(t, nh, dv)
     z = (h @ w[pre + "a1"].T) @ w[pre + "a2"].T + w[pre + "a2.b"]
-    alpha = torch.exp(log_sigmoid(z) / m["tau"]).view(t, nh, d)
-    out = torch.zeros(t, nh, dv, dtype=F64)
-    for a in range(nh):
-        mem = torch.zeros(d, dv, dtype=F64)
-        for s in range(t):
-            mem = alpha[s, a][:, None] * mem + torch.outer(k[s, a], v[s, a])
-            out[s, a] = mem.T @ q[s, a]
+    out = decayed_memory(q, k, v, channel_decay(z, m["tau"]).view(t, nh, d))
     y = unit_rms(out, eps) * w[pre + "norm"]
     return (y.reshape(t, nh * dv) * silu(h @ w[pre + "g"].T)) @ w[pre + "o"].T
 
@@ -112,20 +148,25 @@ def dense_ff(w, pre, h):
     return (gelu_tanh(h @ w[pre + "gate"].T) * (h @ w[pre + "up"].T)) @ w[pre + "down"].T
 
 
-def route(w, pre, h, r):
-    """(chosen ids [T, top], their weights [T, top]); ids >= experts are identity experts."""
-    n = r["experts"] + r.get("identity", 0)
-    s = torch.softmax(h @ w[pre + "router"].T, -1)
-    choice = s + w[pre + "correction"]
-    groups = r.get("groups") or {"count": 1, "keep": 1}
-    per = n // groups["count"]
-    best = choice.view(-1, groups["count"], per).max(-1).values
-    kept = best.topk(groups["keep"], dim=-1).indices
-    allowed = torch.zeros(h.shape[0], groups["count"], dtype=torch.bool)
+def choose(logits, bias, n_groups, keep, top):
+    """Softmax scores; the ``top`` largest of score + bias among the outputs of the ``keep`` groups whose largest
+    biased score is largest -> (ids [T, top], scores of the chosen [T, top])."""
+    s = torch.softmax(logits, -1)
+    choice = s + bias
+    per = logits.shape[1] // n_groups
+    best = choice.view(-1, n_groups, per).max(-1).values
+    kept = best.topk(keep, dim=-1).indices
+    allowed = torch.zeros(logits.shape[0], n_groups, dtype=torch.bool)
     allowed.scatter_(1, kept, True)
     choice = choice.masked_fill(~allowed.repeat_interleave(per, dim=1), -math.inf)
-    ids = choice.topk(r["top"], dim=-1).indices
+    ids = choice.topk(top, dim=-1).indices
     return ids, s.gather(1, ids)
+
+
+def route(w, pre, h, r):
+    """(chosen ids [T, top], their weights [T, top]); ids >= experts are identity experts."""
+    groups = r.get("groups") or {"count": 1, "keep": 1}
+    return choose(h @ w[pre + "router"].T, w[pre + "correction"], groups["count"], groups["keep"], r["top"])
 
 
 def moe_ff(w, pre, h, f):

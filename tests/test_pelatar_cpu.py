@@ -1,0 +1,166 @@
+"""Pelatar on the CPU (the PyTorch definitions of the ops, fp32): every mechanism against its float64
+definition, then the engine (scheduler, pages, state slots, batch assembly, model) against the oracle."""
+
+import json
+import os
+import subprocess
+import sys
+import tempfile
+
+import pytest
+import torch
+
+import pelatar_cases as pc
+import pelatar_oracle as po
+from vllm_production_stack_amd.engine.config import (PRESETS, GatedLinearSpec, MatrixMemorySpec, NormedAttentionSpec,
+                                                     pelatar_layers, resolve_model)
+
+DEV = torch.device("cpu")
+TOL = 2e-5
+
+
+@pytest.fixture(scope="module")
+def model_a():
+    cfg = pc.config_a()
+    return cfg, po.random_weights(cfg, seed=3)
+
+
+@pytest.fixture(scope="module")
+def model_b():
+    cfg = pc.config_b()
+    return cfg, po.random_weights(cfg, seed=4)
+
+
+def test_norm_on_the_sublayer_output():
+    pc.case_norm_on_output(DEV, "float32", 1e-6)
+
+
+def test_gated_units():
+    pc.case_gated_units(DEV, "float32", 1e-5)
+
+
+def test_routing():
+    pc.case_routing(DEV)
+
+
+def test_unit_rms_queries_keys_and_temperature():
+    pc.case_qk_norm(DEV, "float32", 1e-5)
+
+
+def test_attention_with_sink():
+    pc.case_attention(DEV, "float32", 1e-5)
+
+
+def test_matrix_memory():
+    pc.case_matrix_memory(DEV, "float32", 2e-5)
+
+
+def test_decayed_memory():
+    pc.case_decayed_memory(DEV, "float32", 2e-5)
+
+
+def test_config_reader(model_a):
+    cfg, _ = model_a
+    specs = pelatar_layers(json.loads(json.dumps(cfg["layers"])))
+    assert [type(s.mixer) for s in specs] == [MatrixMemorySpec, GatedLinearSpec, NormedAttentionSpec, NormedAttentionSpec]
+    assert specs[3].mixer.kv_from == 2 and specs[2].mixer.temp_every == 16 and specs[1].mlp.identity == 2
+    assert specs[1].mlp.router == "softmax" and specs[0].mlp.act == "gelu_tanh" and specs[0].mlp.gated
+    bad = json.loads(json.dumps(cfg["layers"]))
+    bad[3]["mixer"]["kv_from"] = 1          # not an attention layer
+    with pytest.raises(ValueError):
+        pelatar_layers(bad)
+    bad = json.loads(json.dumps(cfg["layers"]))
+    bad[1]["mlp"]["router"]["groups"]["count"] = 3   # 8 outputs do not split into 3 groups
+    with pytest.raises(ValueError):
+        pelatar_layers(bad)
+    assert PRESETS["tiny-pelatar"].architecture == "pelatar" and PRESETS["tiny-pelatar"].num_params() > 0
+
+
+def test_loader_refuses_what_does_not_fit(model_a):
+    cfg, w = model_a
+    from vllm_production_stack_amd.models.loader import build_model
+
+    def load(weights):
+        folder = po.write_checkpoint(tempfile.mkdtemp(prefix="px-"), cfg, weights)
+        mc, path = resolve_model(str(folder))
+        return build_model(mc, torch.float32, DEV, 256, ckpt_dir=path)
+
+    m = load(w)
+    assert m.layers[1].w_a2.shape[1] == 4       # the decay's low rank came from the checkpoint's tensors
+    missing = {k: v for k, v in w.items() if k != "l2.mix.sink"}
+    with pytest.raises(ValueError):
+        load(missing)
+    with pytest.raises(ValueError):
+        load(dict(w, **{"l3.mix.k": w["l2.mix.k"]}))   # a layer that reads its neighbour's keys has none of its own
+    with pytest.raises(ValueError):
+        load(dict(w, **{"l0.mix.i.b": torch.zeros(3)}))
+
+
+def test_layers_one_by_one(model_a, model_b):
+    pc.check_layers("cpu", "float32", TOL, *model_a)
+    pc.check_layers("cpu", "float32", TOL, *model_b)
+
+
+def test_portions_down_to_one_token(model_a):
+    cfg, w = model_a
+    pc.check_cuts("cpu", "float32", TOL, cfg, w, 140, [[140], [100], [64, 64, 12], [63, 2, 2, 61, 3, 7, 2], [1, 1, 1, 2, 5, 128]])
+
+
+def test_portions_other_sizes(model_b):
+    cfg, w = model_b
+    pc.check_cuts("cpu", "float32", TOL, cfg, w, 150, [[150], [2, 62, 2, 64, 2], [65, 63, 2, 2]], seed=2)
+
+
+def test_recurrences_only():
+    cfg = pc.config_d()
+    w = po.random_weights(cfg, seed=6)
+    pc.check_cuts("cpu", "float32", TOL, cfg, w, 90, [[90], [3, 2, 70], [50]], seed=3)
+
+
+def test_long_decoding(model_b):
+    cfg, w = model_b
+    pc.check_cuts("cpu", "float32", TOL, cfg, w, 200, [[60]], seed=4)   # 140 tokens one by one, across three pages
+
+
+def test_batches_of_unequal_requests(model_a):
+    pc.check_batches("cpu", "float32", TOL, *model_a)
+
+
+def test_a_token_far_back(model_a):
+    cfg, w = model_a
+    pc.check_far_token("cpu", "float32", cfg, w, TOL)
+
+
+def test_generation_through_the_engine(model_a):
+    pc.check_generate("cpu", "float32", *model_a, n_new=6)
+
+
+def test_preemption(model_b):
+    pc.check_preemption("cpu", "float32", *model_b)
+
+
+def test_replay_command(model_a):
+    """The replay program on a checkpoint directory: steps on stdin, logits files, one 'done' line per step."""
+    cfg, w = model_a
+    folder = str(po.write_checkpoint(tempfile.mkdtemp(prefix="px-"), cfg, w))
+    out = tempfile.mkdtemp(prefix="px-out-")
+    toks = pc.tokens(cfg, 70, 9)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:40], "want": [0, 39]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": toks[40:69], "want": []}, {"id": "b", "tokens": toks[:2], "want": [1]}],
+              "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": toks[69:], "want": [0]}], "end": ["a"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                        "--out", out, "--max-tokens", "192", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [ln for ln in r.stdout.splitlines() if ln.startswith("done")] == ["done 0", "done 1", "done 2"]
+    want = po.forward(cfg, w, toks)
+    import numpy as np
+
+    got0 = torch.from_numpy(np.fromfile(os.path.join(out, "0.f32"), dtype="<f4").reshape(2, -1))
+    got1 = torch.from_numpy(np.fromfile(os.path.join(out, "1.f32"), dtype="<f4").reshape(1, -1))
+    got2 = torch.from_numpy(np.fromfile(os.path.join(out, "2.f32"), dtype="<f4").reshape(1, -1))
+    pc.check_rows(got0, want[[0, 39]], TOL, "step 0")
+    pc.check_rows(got1, want[[1]], TOL, "step 1")
+    pc.check_rows(got2, want[[69]], TOL, "step 2")

@@ -492,8 +492,9 @@ def group_topk(logits, experts, groups, keep, topk, route_scale, extra):
 
 def moe_finish(residual, y, weights, pos, shared, gate):
     t, k = weights.shape
-    if k:
-        residual.add_((y[pos.long()].view(t, k, -1).float() * weights[:, :, None]).sum(1))
+    if k:  # a pair of weight 0 is skipped, as in the kernel: its row of y may never have been written
+        rows = torch.where((weights != 0)[:, :, None], y[pos.long()].view(t, k, -1).float(), 0.0)
+        residual.add_((rows * weights[:, :, None]).sum(1))
     if shared is not None:
         residual.add_(shared.float() * (gate[:, None] if gate is not None else 1.0))
     return residual
