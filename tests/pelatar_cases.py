@@ -361,8 +361,9 @@ def case_scan_pieces(dev, dtype, tol):
     for unit in (False, True):
         cols = ops.scan_state_cols(vdim, unit)
         outs, states = [], []
+        start = torch.randn(3, heads * dim * cols + heads, generator=g)   # what the going-on sequences left in their slots
         for pc in (None, pieces):
-            state = torch.randn(3, heads * dim * cols + heads, generator=g).to(dev)
+            state = start.clone().to(dev)
             if unit:
                 prep, _ = ops.mlstm_prepare(proj, 0, hd, logits, zero_h, zero_h, 15.0, heads, dim, 1.0, state,
                                             heads * dim * cols, i32(cu, dev), i32([2, 0, 1], dev), i32(pos, dev))
@@ -407,7 +408,8 @@ def check_rows(got, want, tol, what, loose=0):
     assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} != {tuple(want.shape)}"
     err = po.row_errors(got, want)
     bad = int((err >= tol).sum())
-    assert bad <= loose, f"{what}: {bad} rows off, the worst (row {int(err.argmax())}) by {err.max().item():.3g} (allowed {tol})"
+    loose = max(loose, int(loose / 100 * got.shape[0]))   # from 100 rows on, that many per cent
+    assert err.median().item() < tol and bad <= loose, f"{what}: {bad} rows off, the worst (row {int(err.argmax())}) by {err.max().item():.3g} (allowed {tol})"
     assert torch.isfinite(err).all(), what
 
 
@@ -514,11 +516,12 @@ def check_far_token(device, dtype, cfg, w, tol):
     b[3] = (a[3] + 1) % cfg["vocab"]
     eng = make_engine(cfg, w, device, dtype, pages=12)
     rows = [n - 70, n - 1]
-    outs = []
+    want = {"a": po.forward(cfg, w, a)[rows], "b": po.forward(cfg, w, b)[rows]}
+    assert po.row_errors(want["a"], want["b"]).min().item() > 1e-3          # the early token matters to the answer
     for name, toks in (("a", a), ("b", b)):
         eng.forced_step([(name, toks[:200], [])], [])
         got = eng.forced_step([(name, toks[200:], [r - 200 for r in rows])], [name]).cpu()
-        check_rows(got, po.forward(cfg, w, toks)[rows], tol, f"prompt {name}")
-        outs.append(got)
-    assert po.row_errors(outs[0], outs[1]).min().item() > 10 * tol  # the early token is seen
+        check_rows(got, want[name], tol, f"prompt {name}")
+        other = want["b" if name == "a" else "a"]
+        assert (po.row_errors(got, want[name]) < po.row_errors(got, other)).all()  # and it is seen
     eng.shutdown()

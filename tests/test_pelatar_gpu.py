@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 
 # 16-bit runs: a routing decision that rounding turns over changes a row and says nothing about the kernels, so a few
 # rows may miss the bound there; fp32 is the sharp run
-MODES = [("float32", 5e-5, 0), ("bfloat16", 8e-2, 6)]
+MODES = [("float32", 5e-5, 0), ("bfloat16", 8e-2, 8)]
 KERNEL_TOL = {"float32": 2e-5, "bfloat16": 2e-2}
 DEV = torch.device("cuda")
 

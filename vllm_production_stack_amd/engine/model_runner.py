@@ -360,7 +360,7 @@ class ModelRunner:
             meta.pre_ctx_lens = self._to_dev(plan["pre_ctx"], torch.int32)
             if hasattr(self.model, "plan_prefill"):  # the model's attention kernels take a work list of their own
                 self.model.plan_prefill(meta, q_lens, plan["pre_ctx"], self._to_dev)
-            elif self.device.type == "cuda":
+            elif self.device.type == "cuda" and not hasattr(self.model, "plan_batch"):  # (its kernels have their own lists)
                 rows = ops.prefill_tile_rows(q_lens, self.model.n_q, self.model.n_kv)
                 ts, tq = ops.build_prefill_tiles(q_lens, self.model.n_q, self.model.n_kv, rows, plan["pre_ctx"])
                 cut = ops.plan_prefill_splits(ts, tq, q_lens, plan["pre_ctx"], self.model.n_q, self.model.n_kv, rows)
