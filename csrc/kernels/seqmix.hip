@@ -236,6 +236,9 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
                         : ((unit_col && cc == vsrc) ? 1.f : 0.f);
     }
     __syncthreads();
+    // a wave whose columns all lie past the state's (the last column block of a width that is no multiple of the
+    // block) only helps to stage: its lanes hold zeros that nobody reads
+    if (blockIdx.x * cols + (tid >> 6) * (64 / R) * 4 >= vdim) continue;
     for (int tt = 0; tt < nb; ++tt) {
       const f32x4 v = *reinterpret_cast<const f32x4*>(vs + tt * cols + cb * 4);
       const float* qr = qs + tt * dimp + rg * 4;

@@ -48,7 +48,8 @@
 #define TG_EPI_GLU_CLAMP 3  // paired like SwiGLU: min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, +-limit) + bias)
 #define TG_EPI_RELU_SQ 4    // relu(product)^2
 #define TG_EPI_XIELU 5      // z > 0: act_alpha z^2 + z / 2, else act_bias (exp(z) - 1 - z) + z / 2
-#define TG_PAIRED(E) ((E) == TG_EPI_SWIGLU || (E) == TG_EPI_GLU_CLAMP)
+#define TG_EPI_GELU_GLU 6   // paired like SwiGLU: gelu(g) * u with gelu in its tanh form
+#define TG_PAIRED(E) ((E) == TG_EPI_SWIGLU || (E) == TG_EPI_GLU_CLAMP || (E) == TG_EPI_GELU_GLU)
 
 typedef __attribute__((address_space(3))) void* tg_lds_ptr_t;
 
@@ -308,6 +309,10 @@ __global__ __launch_bounds__(512, 2) void tile_gemm_kernel(
               gt = fminf(gt, act_limit);
               up = fminf(fmaxf(up, -act_limit), act_limit) + act_bias;
               v[4 * ni + e] = gt / (1.f + __expf(-act_alpha * gt)) * up;
+            } else if (EPI == TG_EPI_GELU_GLU) {
+              // 0.5 g (1 + tanh(y)) = g / (1 + exp(-2 y)),  y = sqrt(2 / pi) (g + 0.044715 g^3)
+              const float y2 = 1.5957691216057308f * (gt + 0.044715f * gt * gt * gt);
+              v[4 * ni + e] = gt / (1.f + __expf(-y2)) * up;
             } else {
               v[4 * ni + e] = gt / (1.f + __expf(-gt)) * up;
             }
@@ -368,7 +373,7 @@ VPSA_EXPORT int vpsa_tile_gemm_debug(int v) {
 // output row r reads A row r); w [G, N, K] contiguous; offsets [G + 1] int32 on the device with
 // offsets[G] <= max_rows, or null (one group of max_rows rows); c [max_rows, N] (SwiGLU: N / 2
 // columns), row stride ldc; epi: 0 store, 1 SwiGLU, 2 store of product + resid (row stride ldr; may
-// alias c), 3 clamped gated unit (paired like SwiGLU, constants act_*), 4 squared ReLU, 5 xIELU (act_alpha, act_bias: its two curvatures).  Every byte offset into a and into one group of w must fit 32 bits.
+// alias c), 6 gated gelu unit (tanh form, paired like SwiGLU), 3 clamped gated unit (paired like SwiGLU, constants act_*), 4 squared ReLU, 5 xIELU (act_alpha, act_bias: its two curvatures).  Every byte offset into a and into one group of w must fit 32 bits.
 // Returns 0, or a negative number when the shape is outside what the kernel tiles.
 VPSA_EXPORT int vpsa_tile_gemm(const void* a, long lda, const void* arow_idx, const void* w, const void* offsets,
                                int n_groups, void* c, long ldc, int max_rows, int n, int k, int epi, const void* resid,
@@ -379,7 +384,7 @@ VPSA_EXPORT int vpsa_tile_gemm(const void* a, long lda, const void* arow_idx, co
   if (TG_PAIRED(epi) && (n % 2 != 0 || (n / 2) % 32 != 0)) return -1;
   if (!TG_PAIRED(epi) && n % 8 != 0) return -1;
   if (epi == TG_EPI_RESIDUAL && (!resid || ldr % 8 != 0)) return -1;
-  if (epi < 0 || epi > 5) return -1;
+  if (epi < 0 || epi > 6) return -1;
   if ((double)a_rows * (double)lda * 2.0 >= 4294967296.0 || (double)n * (double)k * 2.0 >= 4294967296.0) return -1;
   const int n_tiles = TG_PAIRED(epi) ? (n / 2 + 127) / 128 : (n + TG_BN - 1) / TG_BN;
   const int m_tiles_max = offsets ? max_rows / TG_BM + n_groups : (max_rows + TG_BM - 1) / TG_BM;
@@ -404,6 +409,7 @@ VPSA_EXPORT int vpsa_tile_gemm(const void* a, long lda, const void* arow_idx, co
   else if (epi == TG_EPI_GLU_CLAMP) TG_LAUNCH(TG_EPI_GLU_CLAMP, 0);
   else if (epi == TG_EPI_RELU_SQ) TG_LAUNCH(TG_EPI_RELU_SQ, 0);
   else if (epi == TG_EPI_XIELU) TG_LAUNCH(TG_EPI_XIELU, 0);
+  else if (epi == TG_EPI_GELU_GLU) TG_LAUNCH(TG_EPI_GELU_GLU, 0);
   else if (g_tg_debug == 1) TG_LAUNCH(TG_EPI_PLAIN, 1);
   else if (g_tg_debug == 2) TG_LAUNCH(TG_EPI_PLAIN, 2);
   else if (g_tg_debug == 3) TG_LAUNCH(TG_EPI_PLAIN, 3);

@@ -103,6 +103,11 @@ def case_gated_units(dev, dtype, tol):
     h = torch.randn(5, 40, generator=g).to(dt)
     want = po.gelu_tanh(h.double() @ w[:24].double().T) * (h.double() @ w[24:].double().T)
     close(ops.gate_up_act(h.to(dev), w.to(dev), "gelu_tanh"), want, max(tol, 2e-2 if dt == torch.bfloat16 else 0), "fused projection")
+    if dt == torch.bfloat16 and torch.device(dev).type == "cuda":  # the same unit in the prefill GEMM's epilogue
+        w = (torch.randn(2 * 96, 128, generator=g) * 0.3).to(dt)
+        h = torch.randn(300, 128, generator=g).to(dt)
+        want = po.gelu_tanh(h.double() @ w[:96].double().T) * (h.double() @ w[96:].double().T)
+        close(ops.tile_gemm(h.to(dev), w.to(dev), gelu_mul=True), want, 2e-2, "epilogue of the prefill GEMM")
 
 
 def case_routing(dev):

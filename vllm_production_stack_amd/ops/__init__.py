@@ -731,7 +731,7 @@ TILE_CUS = 256
 _tile_enabled = os.environ.get("VPSA_TILE_GEMM", "1") != "0"
 
 
-TILE_GELU_GLU = False  # the gated gelu unit in the prefill GEMM's epilogue (tile_gemm(gelu_mul=True))
+TILE_GELU_GLU = True  # the gated gelu unit in the prefill GEMM's epilogue (tile_gemm(gelu_mul=True))
 
 
 def set_tile_gemm(on: bool) -> bool:
@@ -1195,7 +1195,7 @@ def tile_gemm_supported(n: int, k: int, silu_mul: bool = False) -> bool:
 
 
 def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, residual=None, out=None, glu_clamp=None,
-              relu_sq=False, xielu=None):
+              relu_sq=False, xielu=None, gelu_mul=False):
     """The prefill GEMM (``csrc/kernels/tile_gemm.hip``): out[r] = epilogue(a[arow_idx[r] or r] @ w[g]^T).
 
     a [*, K] bf16; w [N, K] (dense) or [G, N, K] (grouped, with offsets [G + 1] int32 ON THE DEVICE:
@@ -1204,8 +1204,9 @@ def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, resi
     residual (``out`` may be ``residual`` itself).  glu_clamp = (limit, alpha, bias): w is [gate rows | up
     rows] as for silu_mul, out = min(g, limit) * sigmoid(alpha min(g, limit)) * (clamp(u, +-limit) + bias).
     relu_sq: out = relu(product)^2.  xielu = (a_pos, a_neg): out = a_pos z^2 + z / 2 for z > 0, else
-    a_neg (exp(z) - 1 - z) + z / 2.  Rows at or past offsets[G] are left unwritten."""
-    paired = silu_mul or glu_clamp is not None
+    a_neg (exp(z) - 1 - z) + z / 2.  gelu_mul: paired like silu_mul, out = gelu(gate) * up with gelu in its tanh
+    form.  Rows at or past offsets[G] are left unwritten."""
+    paired = silu_mul or glu_clamp is not None or gelu_mul
     if w.dim() == 2:
         w = w.unsqueeze(0)
     g, n, k = w.shape
@@ -1214,7 +1215,7 @@ def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, resi
     n_out = n // 2 if paired else n
     _bf16_cuda(a, w, residual)
     assert w.is_contiguous() and a.stride(-1) == 1 and a.shape[1] == k
-    assert sum((silu_mul, glu_clamp is not None, relu_sq, residual is not None, xielu is not None)) <= 1
+    assert sum((silu_mul, glu_clamp is not None, relu_sq, residual is not None, xielu is not None, gelu_mul)) <= 1
     if offsets is not None:
         assert offsets.dtype == torch.int32 and offsets.numel() == g + 1 and offsets.is_cuda
     else:
@@ -1230,6 +1231,8 @@ def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, resi
     lim, alpha, bias = glu_clamp if glu_clamp is not None else (0.0, 1.0, 0.0)
     if xielu is not None:
         epi, alpha, bias = 5, float(xielu[0]), float(xielu[1])
+    if gelu_mul:
+        epi = 6
     rc = _kernels().vpsa_tile_gemm(_p(a), c_long(a.stride(0)), _p(arow_idx), _p(w), _p(offsets), c_int(g), _p(out),
                                    c_long(out.stride(0)), c_int(rows), c_int(n), c_int(k), c_int(epi), _p(residual),
                                    c_long(residual.stride(0) if residual is not None else 0), c_long(a.shape[0]),

@@ -302,8 +302,12 @@ def gate_up_act(x, w_gate_up, act: str, packed=None):
     if act == "silu" and x.is_cuda and x.dtype == torch.bfloat16:
         return o.gate_up_silu(x, w_gate_up, packed)
     rows = o.tile_rows(x, w_gate_up, True) if (x.is_cuda and act == "gelu_tanh" and o.TILE_GELU_GLU) else 0
-    if rows == x.shape[0] and rows:
-        return o.tile_gemm(x, w_gate_up, gelu_mul=True)
+    if rows:
+        out = torch.empty((x.shape[0], w_gate_up.shape[0] // 2), dtype=x.dtype, device=x.device)
+        o.tile_gemm(x[:rows], w_gate_up, gelu_mul=True, out=out[:rows])
+        if rows < x.shape[0]:
+            out[rows:] = glu_act(o.linear(x[rows:], w_gate_up), act)
+        return out
     return glu_act(o.linear(x, w_gate_up), act)
 
 
