@@ -212,7 +212,7 @@ def forward(cfg, weights, tokens, probe=None):
 
 
 # ----------------------------------------------------------------------------- configurations and weights for tests
-def attention_layer(heads=4, kv_heads=2, dim=16, vdim=24, scale=None, coef=0.5, every=16, kv_from=None, mlp=None):
+def attention_layer(heads=4, kv_heads=2, dim=16, vdim=24, scale=None, coef=0.4, every=16, kv_from=None, mlp=None):
     m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale if scale is not None else dim ** -0.5}
     if coef:
         m["q_temp"] = {"coef": coef, "every": every}
@@ -221,11 +221,11 @@ def attention_layer(heads=4, kv_heads=2, dim=16, vdim=24, scale=None, coef=0.5, 
     return {"type": "attention", "mixer": m, "mlp": mlp}
 
 
-def mlstm_layer(heads=2, dim=16, vdim=24, cap=15.0, mlp=None):
+def mlstm_layer(heads=2, dim=16, vdim=24, cap=12.0, mlp=None):
     return {"type": "mlstm", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "gate_cap": cap}, "mlp": mlp}
 
 
-def gla_layer(heads=2, dim=16, vdim=24, tau=16.0, rank=8, mlp=None):
+def gla_layer(heads=2, dim=16, vdim=24, tau=8.0, rank=8, mlp=None):
     # the rank is no key of the configuration: the shape of the first decay projection carries it
     return {"type": "gla", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau}, "mlp": mlp, "_rank": rank}
 

@@ -117,6 +117,11 @@ def test_recurrences_only():
     pc.check_cuts("cpu", "float32", TOL, cfg, w, 90, [[90], [3, 2, 70], [50]], seed=3)
 
 
+def test_sizes_that_are_multiples_of_nothing():
+    cfg = pc.config_f()
+    pc.check_cuts("cpu", "float32", TOL, cfg, po.random_weights(cfg, seed=8), 100, [[100], [66, 2, 1, 20], [1, 1, 3]])
+
+
 def test_long_decoding(model_b):
     cfg, w = model_b
     pc.check_cuts("cpu", "float32", TOL, cfg, w, 200, [[60]], seed=4)   # 140 tokens one by one, across three pages

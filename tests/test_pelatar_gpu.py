@@ -110,6 +110,22 @@ def test_tiled_kernels_and_pieces_in_the_engine(dtype, tol, loose, model_c):
 
 
 @pytest.mark.parametrize("dtype,tol,loose", MODES)
+def test_decode_sized_mixture_kernels(dtype, tol, loose):
+    cfg = pc.config_e()
+    assert ops.moe_mfma_supported(128, 512)
+    pc.check_cuts("cuda", dtype, tol, cfg, po.random_weights(cfg, seed=7), 120, [[120], [70, 40, 3], [30, 2, 2]], loose=loose)
+
+
+@pytest.mark.parametrize("dtype,tol,loose", MODES)
+def test_sizes_that_are_multiples_of_nothing(dtype, tol, loose):
+    cfg = pc.config_f()
+    tol = tol if dtype == "float32" else 0.15   # a width of 20 averages bf16 rounding over few terms
+    pc.check_cuts("cuda", dtype, tol, cfg, po.random_weights(cfg, seed=8), 100, [[100], [66, 2, 1, 20], [1, 1, 3]], loose=loose)
+    if dtype == "float32":  # (in 16 bits a width of 20 turns routing decisions over in too many rows to say anything)
+        pc.check_batches("cuda", dtype, tol, cfg, po.random_weights(cfg, seed=8))
+
+
+@pytest.mark.parametrize("dtype,tol,loose", MODES)
 def test_recurrences_only(dtype, tol, loose):
     cfg = pc.config_d()
     tol = tol if dtype == "float32" else 0.15   # a width of 24 averages bf16 rounding over few terms

@@ -655,9 +655,9 @@ def _px_moe(ff, experts, top, groups, keep, identity):
             "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}, "identity": identity}}
 
 
-def _px_attention(heads, kv_heads, dim, vdim, mlp=None, kv_from=None, every=128):
+def _px_attention(heads, kv_heads, dim, vdim, mlp=None, kv_from=None, every=256):
     m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
-         "q_temp": {"coef": 0.5, "every": every}}
+         "q_temp": {"coef": 0.4, "every": every}}
     if kv_from is not None:
         m["kv_from"] = kv_from
     return {"type": "attention", "mixer": m, "mlp": mlp}
@@ -670,8 +670,8 @@ def pelatar_stack(width, heads, ff, experts, unit_ff, top, identity, blocks=1):
     routed = _px_moe(unit_ff, experts, top, 4, 2, identity)
     out = []
     for b in range(blocks):
-        out += [{"type": "mlstm", "mlp": dense, "mixer": {"heads": heads // 2, "dim": 128, "vdim": 256, "gate_cap": 15.0}},
-                {"type": "gla", "mlp": routed, "mixer": {"heads": heads // 2, "dim": 128, "vdim": 256, "tau": 16.0}},
+        out += [{"type": "mlstm", "mlp": dense, "mixer": {"heads": heads // 2, "dim": 128, "vdim": 256, "gate_cap": 12.0}},
+                {"type": "gla", "mlp": routed, "mixer": {"heads": heads // 2, "dim": 128, "vdim": 256, "tau": 8.0}},
                 _px_attention(heads, heads // 4, 128, 128, dense),
                 _px_attention(heads, heads // 4, 128, 128, routed, kv_from=4 * b + 2)]
     return out
@@ -680,8 +680,8 @@ def pelatar_stack(width, heads, ff, experts, unit_ff, top, identity, blocks=1):
 # Pelatar at random weights: a small one for smoke runs, and one with layer shapes of a 2048-wide model
 PRESETS["tiny-pelatar"] = pelatar_config(
     "tiny-pelatar", 512, 128,
-    [{"type": "mlstm", "mlp": {"kind": "dense", "ff": 256}, "mixer": {"heads": 2, "dim": 32, "vdim": 64, "gate_cap": 15.0}},
-     {"type": "gla", "mlp": _px_moe(64, 6, 2, 2, 1, 2), "mixer": {"heads": 2, "dim": 64, "vdim": 32, "tau": 16.0}},
+    [{"type": "mlstm", "mlp": {"kind": "dense", "ff": 256}, "mixer": {"heads": 2, "dim": 32, "vdim": 64, "gate_cap": 12.0}},
+     {"type": "gla", "mlp": _px_moe(64, 6, 2, 2, 1, 2), "mixer": {"heads": 2, "dim": 64, "vdim": 32, "tau": 8.0}},
      _px_attention(4, 2, 64, 128, {"kind": "dense", "ff": 256}, every=64),
      _px_attention(4, 2, 64, 128, _px_moe(64, 4, 2, 1, 1, 0), kv_from=2, every=64)], max_position_embeddings=4096)
 PRESETS["pelatar-bench"] = pelatar_config("pelatar-bench", 32000, 2048, pelatar_stack(2048, 16, 5632, 28, 1024, 4, 4),
