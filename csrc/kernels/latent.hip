@@ -291,7 +291,8 @@ __global__ __launch_bounds__(256) void glu_clamp_kernel(const T* __restrict__ x,
 __global__ __launch_bounds__(64) void group_topk_kernel(const float* __restrict__ logits, int cols,
                                                         float* __restrict__ weights, int* __restrict__ ids,
                                                         float* __restrict__ extra_out, int experts, int groups,
-                                                        int keep, int topk, float route_scale) {
+                                                        int keep, int topk, float route_scale, int normalize) {
+  // normalize: the chosen scores are divided by their sum (+ 1e-20) before route_scale
   __shared__ float s[ROUTE_MAX_EXPERTS];
   __shared__ float gs[ROUTE_MAX_EXPERTS];
   const long t = blockIdx.x;
@@ -337,6 +338,12 @@ __global__ __launch_bounds__(64) void group_topk_kernel(const float* __restrict_
     __syncthreads();
     if (lane == 0) s[bi] = -3.f;
     __syncthreads();
+  }
+  if (normalize && lane == 0) {
+    float sum = 0.f;
+    for (int k = 0; k < topk; ++k) sum += weights[t * topk + k];
+    const float inv = 1.f / (sum / route_scale + 1e-20f);
+    for (int k = 0; k < topk; ++k) weights[t * topk + k] *= inv;
   }
 }
 
@@ -434,6 +441,54 @@ __global__ __launch_bounds__(256) void rmsnorm_add_kernel(float* __restrict__ re
     r[i] = v;
     if (y) Conv<T>::st(y + row * n + i, v);
   }
+}
+
+// A gated residual in front of a pre-norm.  Per row:
+//   residual += sigmoid(gate + gate_bias) (.) (c1 n1(d1) + c2 n2(d2)) + extra + extra_vec;  y = rmsnorm(residual) w
+// with n_i(d) = rmsnorm(d) w_i where a weight w_i is given and d itself otherwise.  Every part is optional: no gate
+// means a plain add, no deltas only the extras (a second stream that re-enters, a vector per pass of a layer loop).
+// d1 in D (the activation dtype, or fp32 for a mixture's sum), d2, gate and y in T.
+template <typename T, typename D>
+__global__ __launch_bounds__(256) void gated_add_rmsnorm_kernel(
+    float* __restrict__ residual, const D* __restrict__ d1, long s1, const float* __restrict__ w1, float c1,
+    const T* __restrict__ d2, long s2, const float* __restrict__ w2, float c2, const T* __restrict__ gate, long sg,
+    const float* __restrict__ gate_bias, const float* __restrict__ extra, const float* __restrict__ extra_vec,
+    const float* __restrict__ w, T* __restrict__ y, int n, float eps) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  float* r = residual + row * n;
+  float f1 = c1, f2 = c2;
+  if (d1 && w1) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += 256) {
+      const float v = Conv<D>::ld(d1 + row * s1 + i);
+      ss += v * v;
+    }
+    f1 = c1 / sqrtf(block_sum(ss, red) / (float)n + eps);
+  }
+  if (d2 && w2) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += 256) {
+      const float v = Conv<T>::ld(d2 + row * s2 + i);
+      ss += v * v;
+    }
+    f2 = c2 / sqrtf(block_sum(ss, red) / (float)n + eps);
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    float d = 0.f;
+    if (d1) d += Conv<D>::ld(d1 + row * s1 + i) * f1 * (w1 ? w1[i] : 1.f);
+    if (d2) d += Conv<T>::ld(d2 + row * s2 + i) * f2 * (w2 ? w2[i] : 1.f);
+    if (gate) d *= sigmoidf(Conv<T>::ld(gate + row * sg + i) + (gate_bias ? gate_bias[i] : 0.f));
+    float v = r[i] + d;
+    if (extra) v += extra[row * n + i];
+    if (extra_vec) v += extra_vec[i];
+    r[i] = v;  // read back below by the same thread
+    ss += v * v;
+  }
+  if (!y) return;
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += 256) Conv<T>::st(y + row * n + i, r[i] * inv * w[i]);
 }
 
 // x [rows, 2 inter] = gate | up  ->  act(gate) * up;  kind 0: silu, 1: gelu in its tanh form
@@ -588,13 +643,31 @@ VPSA_EXPORT int vpsa_glu_clamp(const void* x, long x_stride, void* y, int rows, 
 
 VPSA_EXPORT int vpsa_group_topk(const float* logits, int cols, float* weights, int* ids, float* extra_out,
                                 int tokens, int experts, int groups, int keep, int topk, float route_scale,
-                                hipStream_t st) {
+                                int normalize, hipStream_t st) {
   if (tokens <= 0) return 0;
   if (experts > ROUTE_MAX_EXPERTS || groups < 1 || experts % groups || keep < 1 || keep > groups ||
       topk > experts / groups * keep || cols < experts + (extra_out ? 1 : 0))
     return -1;
   hipLaunchKernelGGL(group_topk_kernel, dim3(tokens), dim3(64), 0, st, logits, cols, weights, ids, extra_out,
-                     experts, groups, keep, topk, route_scale);
+                     experts, groups, keep, topk, route_scale, normalize);
+  return 0;
+}
+
+// d1_f32: the first delta is fp32 whatever the activation dtype (a mixture's fp32 sum)
+VPSA_EXPORT int vpsa_gated_add_rmsnorm(float* residual, const void* d1, long s1, int d1_f32, const float* w1, float c1,
+                                       const void* d2, long s2, const float* w2, float c2, const void* gate, long sg,
+                                       const float* gate_bias, const float* extra, const float* extra_vec,
+                                       const float* w, void* y, int rows, int n, float eps, int dtype, hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (dtype != 0 && dtype != 1) return -2;
+  if (y && !w) return -1;
+#define GA(T, D)                                                                                                     \
+  gated_add_rmsnorm_kernel<T, D><<<rows, 256, 0, st>>>(residual, (const D*)d1, s1, w1, c1, (const T*)d2, s2, w2, c2, \
+                                                       (const T*)gate, sg, gate_bias, extra, extra_vec, w, (T*)y, n, eps)
+  if (dtype == 1) GA(float, float);
+  else if (d1_f32) GA(bf16_t, float);
+  else GA(bf16_t, bf16_t);
+#undef GA
   return 0;
 }
 

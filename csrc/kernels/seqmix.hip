@@ -113,7 +113,8 @@ __global__ __launch_bounds__(256) void scan_prepare_kernel(const T* __restrict__
                                                            const float* __restrict__ cos_sin, int rot_dims, int layout,
                                                            float k_scale, const float* __restrict__ gate_bias,
                                                            const float* __restrict__ gate_lower,
-                                                           float* __restrict__ prep) {
+                                                           float* __restrict__ prep, int qk_act) {
+  // qk_act (fixed decay): q and k pass through silu before the rotation
   constexpr int NP = GATED ? 3 : 2;
   const long row = blockIdx.x;
   const T* qp = proj + row * p_stride + q_col;
@@ -133,8 +134,9 @@ __global__ __launch_bounds__(256) void scan_prepare_kernel(const T* __restrict__
     } else {
       const T* qh = qp + h * dim;
       const T* kh = kp + h * dim;
-      d[0] = rotated([&](int c) { return Cv<T>::ld(qh + c); }, i, cs, rot_dims, layout);
-      d[dim] = rotated([&](int c) { return Cv<T>::ld(kh + c); }, i, cs, rot_dims, layout) * k_scale;
+      auto act = [&](float x) { return qk_act ? x * sigm(x) : x; };
+      d[0] = rotated([&](int c) { return act(Cv<T>::ld(qh + c)); }, i, cs, rot_dims, layout);
+      d[dim] = rotated([&](int c) { return act(Cv<T>::ld(kh + c)); }, i, cs, rot_dims, layout) * k_scale;
     }
   }
 }
@@ -156,7 +158,8 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
     const T* __restrict__ proj, long p_stride, int v_col, int heads, int dim, int vdim, const float* __restrict__ prep,
     float* __restrict__ state, long state_stride, const int* __restrict__ seq_cu, const int* __restrict__ seq_state,
     const int* __restrict__ positions, const float* __restrict__ decay, float* __restrict__ out, int R, int TB,
-    const int* __restrict__ pieces, float* __restrict__ ws_state, int vsrc, int unit_col) {
+    const int* __restrict__ pieces, float* __restrict__ ws_state, int vsrc, int unit_col, int v_act) {
+  // v_act: values pass through silu on their way in
   // vsrc: value columns per head that `proj` holds (vdim, or one less than the state's columns need when
   // unit_col: column vsrc of every token's value is then 1 and columns past it are 0)
   constexpr int NP = GATED ? 3 : 2;
@@ -232,8 +235,10 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
     for (int e = tid; e < nb * cols; e += 256) {
       const int tt = e / cols, c = e - tt * cols;
       const int cc = blockIdx.x * cols + c;
-      vs[e] = cc < vsrc ? Cv<T>::ld(proj + (long)(rb + tt) * p_stride + v_col + head * vsrc + cc)
-                        : ((unit_col && cc == vsrc) ? 1.f : 0.f);
+      float x = cc < vsrc ? Cv<T>::ld(proj + (long)(rb + tt) * p_stride + v_col + head * vsrc + cc)
+                          : ((unit_col && cc == vsrc) ? 1.f : 0.f);
+      if (v_act) x = x * sigm(x);
+      vs[e] = x;
     }
     __syncthreads();
     // a wave whose columns all lie past the state's (the last column block of a width that is no multiple of the
@@ -457,17 +462,22 @@ __global__ __launch_bounds__(256) void mlstm_prepare_kernel(const T* __restrict_
   }
 }
 
-// One workgroup per row, a wave per head in turn.  Row = q [heads * dim] (| k [kv_heads * dim] | v [kv_heads * vdim]
+// One workgroup per row, a wave per head in turn.  Row = q [heads * dim] (| k [kv_heads * dim] | v [v_heads * vdim]
 // when the layer owns its cache entries).  q and k heads are divided by their root mean square (eps inside the
-// root, no weight); q is then multiplied by 1 + coef ln(floor((p + 1) / every) + 1) at position p.  k and v go to
-// the page layout of window_attention (K key by key, V transposed).
+// root), multiplied by a weight per channel where one is given (qw / kw, shared by the heads), and turned by the
+// rotary table over their first rot_dims channels (cos_sin null: no rotation); q is then multiplied by
+// 1 + coef ln(floor((p + 1) / every) + 1) at position p.  k and v go to the page layout of window_attention
+// (K key by key, V transposed); designs with several key maps per value head have fewer value heads than key heads.
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_write_kernel(const T* __restrict__ proj, long p_stride, int heads,
                                                             int kv_heads, int dim, int vdim, int own,
                                                             const int* __restrict__ positions,
                                                             const long* __restrict__ slots, float eps, float coef,
                                                             float every, T* __restrict__ q_out, T* __restrict__ cache,
-                                                            long page_stride) {
+                                                            long page_stride, int v_heads,
+                                                            const float* __restrict__ qw, const float* __restrict__ kw,
+                                                            const float* __restrict__ cos_sin, int rot_dims,
+                                                            int layout) {
   const long row = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* pr = proj + row * p_stride;
@@ -485,18 +495,79 @@ __global__ __launch_bounds__(256) void qk_norm_write_kernel(const T* __restrict_
     }
     ss = wave_reduce_sum(ss);
     const float inv = 1.f / sqrtf(ss / (float)dim + eps);
+    const float* w = hh < heads ? qw : kw;
+    const float* cs = cos_sin ? cos_sin + (long)p * rot_dims : nullptr;
+    auto normed = [&](int c) { return Cv<T>::ld(src + c) * inv * (w ? w[c] : 1.f); };
+    auto value = [&](int i) { return cs ? rotated(normed, i, cs, rot_dims, layout) : normed(i); };
     if (hh < heads) {
-      for (int i = lane; i < dim; i += 64) Cv<T>::st(q_out + (row * heads + hh) * dim + i, Cv<T>::ld(src + i) * inv * temp);
+      for (int i = lane; i < dim; i += 64) Cv<T>::st(q_out + (row * heads + hh) * dim + i, value(i) * temp);
     } else if (slot >= 0) {
       T* dst = cache + (slot / PAGE) * page_stride + (slot % PAGE) * nk + (long)(hh - heads) * dim;
-      for (int i = lane; i < dim; i += 64) Cv<T>::st(dst + i, Cv<T>::ld(src + i) * inv);
+      for (int i = lane; i < dim; i += 64) Cv<T>::st(dst + i, value(i));
     }
   }
   if (slot >= 0) {
     const T* vs = pr + (long)heads * dim + nk;
     T* dst = cache + (slot / PAGE) * page_stride + (long)PAGE * nk + (slot % PAGE);
-    for (int c = threadIdx.x; c < kv_heads * vdim; c += 256) dst[(long)c * PAGE] = vs[c];
+    for (int c = threadIdx.x; c < v_heads * vdim; c += 256) dst[(long)c * PAGE] = vs[c];
   }
+}
+
+// Pooled entries of a windowed attention that also sees a mean key and value per block of `pool` tokens.  One
+// workgroup per row of the step: a row at position p with (p + 1) % pool == 0 completes block b = p / pool; the
+// block's keys and values are read back from the pages (as the cache holds them, whichever step wrote them), summed
+// in position order in fp32 and divided by pool, and stored as entry b % PAGE of the pooled region (pool_off
+// elements behind the token region, same layout) of the sequence's page b / PAGE.
+template <typename T>
+__global__ __launch_bounds__(256) void pool_blocks_kernel(T* __restrict__ cache, long page_stride, long pool_off,
+                                                          const int* __restrict__ block_tables, int bt_stride,
+                                                          const int* __restrict__ row_seq,
+                                                          const int* __restrict__ positions,
+                                                          const long* __restrict__ slots, int nk, int nv, int pool) {
+  const long row = blockIdx.x;
+  const int p = positions[row];
+  if (slots[row] < 0 || (p + 1) % pool != 0) return;
+  const int seq = row_seq ? row_seq[row] : (int)row;
+  const int* bt = block_tables + (long)seq * bt_stride;
+  const int b = p / pool, j0 = b * pool;
+  T* dst = cache + (long)bt[b / PAGE] * page_stride + pool_off;
+  const float inv = 1.f / (float)pool;
+  for (int c = threadIdx.x; c < nk + nv; c += 256) {
+    float acc = 0.f;
+    for (int j = j0; j <= p; ++j) {
+      const T* src = cache + (long)bt[j / PAGE] * page_stride;
+      acc += c < nk ? Cv<T>::ld(src + (long)(j % PAGE) * nk + c)
+                    : Cv<T>::ld(src + (long)PAGE * nk + (long)(c - nk) * PAGE + j % PAGE);
+    }
+    if (c < nk) Cv<T>::st(dst + (long)(b % PAGE) * nk + c, acc * inv);
+    else Cv<T>::st(dst + (long)PAGE * nk + (long)(c - nk) * PAGE + b % PAGE, acc * inv);
+  }
+}
+
+// Differential attention's combination.  u fp32 [rows, 2 heads, vdim]: per key/value group g of `rep` query heads the
+// first map's outputs of its heads, then the second map's ([g][map][head in group]).  One wave per (row, head):
+// o = a1 - lambda a2, divided by its root mean square over vdim (eps inside the root), times post; y [rows, heads * vdim]
+// with the heads in their natural order.
+template <typename T>
+__global__ __launch_bounds__(256) void diff_heads_kernel(const float* __restrict__ u, T* __restrict__ y, long pairs,
+                                                         int heads, int rep, int vdim, float lambda, float eps,
+                                                         float post) {
+  const long pair = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= pairs) return;
+  const int lane = threadIdx.x & 63;
+  const long row = pair / heads;
+  const int head = (int)(pair - row * heads);
+  const int g = head / rep, j = head - g * rep;
+  const float* a1 = u + ((row * 2 * heads) + (long)g * 2 * rep + j) * vdim;
+  const float* a2 = a1 + (long)rep * vdim;
+  float ss = 0.f;
+  for (int c = lane; c < vdim; c += 64) {
+    const float v = a1[c] - lambda * a2[c];
+    ss += v * v;
+  }
+  ss = wave_reduce_sum(ss);
+  const float inv = post / sqrtf(ss / (float)vdim + eps);
+  for (int c = lane; c < vdim; c += 64) Cv<T>::st(y + pair * vdim + c, (a1[c] - lambda * a2[c]) * inv);
 }
 
 // One wave per (row, head).  o [pairs][ostride] fp32, of which the first vdim columns are the head's output.
@@ -619,18 +690,34 @@ __global__ __launch_bounds__(256) void conv_tail_kernel(const T* __restrict__ pr
 // Layer cache inside a page: K [PAGE][kv_heads * dim], then V transposed [kv_heads * vdim][PAGE].
 // The pages a query at position p (or a tile of queries p_a .. p_b) has to visit: those that hold kept first
 // tokens below the window, then the window's own; the mask decides key by key.
+// mode 1: `window` is a chunk size instead, and a query sees the keys of its own chunk (chunks counted from
+// position 0) up to itself.
+// pool > 0: beside its window a query at position p sees one pooled entry per block of `pool` tokens that lies
+// wholly before the window, blocks 0 .. seen_blocks(p) - 1.  Block b's entry is entry b % PAGE of the pooled region
+// of the sequence's page b / PAGE (same layout as the token region, pool_off elements behind it); the walk visits
+// those pages first (its first n_keep visits, `pooled`), then the window's.  keep_first is 0 then.
+__device__ __forceinline__ int seen_blocks(int p, int window, int pool) {
+  const int a = p - window + 1;  // tokens before the window
+  return a > 0 ? a / pool : 0;
+}
+
 struct PageWalk {
   int n_keep, first, count;
-  __device__ __forceinline__ PageWalk(int pa, int pb, int window, int keep_first) {
-    const int lo = max(0, pa - window + 1);
+  bool pool_walk;
+  __device__ __forceinline__ PageWalk(int pa, int pb, int window, int keep_first, int mode = 0, int pool = 0) {
+    const int lo = mode == 1 ? pa - pa % window : max(0, pa - window + 1);
     first = lo / PAGE;
-    n_keep = min((min(keep_first, lo) + PAGE - 1) / PAGE, first);
+    pool_walk = pool > 0;
+    if (pool_walk) n_keep = (seen_blocks(pb, window, pool) + PAGE - 1) / PAGE;
+    else n_keep = min((min(keep_first, lo) + PAGE - 1) / PAGE, first);
     count = n_keep + pb / PAGE - first + 1;
   }
   __device__ __forceinline__ int page(int i) const { return i < n_keep ? i : first + (i - n_keep); }
+  __device__ __forceinline__ bool pooled(int i) const { return pool_walk && i < n_keep; }
 };
 
-__device__ __forceinline__ bool key_seen(int j, int p, int window, int keep_first) {
+__device__ __forceinline__ bool key_seen(int j, int p, int window, int keep_first, int mode = 0) {
+  if (mode == 1) return j <= p && j >= p - p % window;
   return j <= p && (p - j < window || j < keep_first);
 }
 
@@ -646,8 +733,10 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
     const T* __restrict__ q, long q_stride, const T* __restrict__ cache, long page_stride,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ row_seq,
     const int* __restrict__ positions, const float* __restrict__ sink, float* __restrict__ out, int heads, int kv_heads,
-    int dim, int vdim, int window, int keep_first, float scale, float softcap, int own) {
+    int dim, int vdim, int window, int keep_first, float scale, float softcap, int own, int mode, int pool,
+    long pool_off, int maps) {
   // own: only the values of the head's own KV head (out [rows, heads, vdim]); designs without head mixing
+  // maps: key heads per value head (kv_heads counts key heads; key head g reads the values of head g / maps)
   extern __shared__ float sm[];
   __shared__ float red[4];
   __shared__ float ps[WA_KEYS];
@@ -659,11 +748,12 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
   const int seq = row_seq ? row_seq[row] : (int)row;
   const int pos = positions[row];
   const int g = head / (heads / kv_heads);
-  const int nk = kv_heads * dim, nv = own ? vdim : kv_heads * vdim;
-  const int c0 = own ? g * vdim : 0;  // first value channel this head reads
+  const int nk = kv_heads * dim, nv = own ? vdim : kv_heads / maps * vdim;
+  const int c0 = own ? g / maps * vdim : 0;  // first value channel this head reads
+  const int nb = pool > 0 ? seen_blocks(pos, window, pool) : 0;
   float* qs = sm;
   for (int i = tid; i < dim; i += 256) qs[i] = Cv<T>::ld(q + row * q_stride + head * dim + i);
-  const PageWalk walk(pos, pos, window, keep_first);
+  const PageWalk walk(pos, pos, window, keep_first, mode, pool);
   const int* bt = block_tables + (long)seq * bt_stride;
   float m = sink ? sink[head] : -INFINITY, l = sink ? 1.f : 0.f;
   float acc[WA_ACC];
@@ -675,10 +765,11 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
     float s = -INFINITY;
     if (pi < walk.count) {
       const int pg = walk.page(pi);
-      const long base = (long)bt[pg] * page_stride;
+      const bool pooled = walk.pooled(pi);
+      const long base = (long)bt[pg] * page_stride + (pooled ? pool_off : 0);
       if (r == 0) pbase[tid / PAGE] = base;
       const int j = pg * PAGE + r;
-      if (key_seen(j, pos, window, keep_first)) {
+      if (pooled ? j < nb : key_seen(j, pos, window, keep_first, mode)) {
         const T* kp = cache + base + (long)r * nk + g * dim;
         float d = 0.f;
         for (int i = 0; i < dim; ++i) d = fmaf(qs[i], Cv<T>::ld(kp + i), d);
@@ -740,7 +831,8 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles,
     const int* __restrict__ positions, const float* __restrict__ sink, float* __restrict__ out, int heads, int kv_heads,
     int window, int keep_first, float scale, float softcap, int splits, float* __restrict__ ws_o,
-    float* __restrict__ ws_ml, int n_chunks, int own) {
+    float* __restrict__ ws_ml, int n_chunks, int own, int mode, int pool, long pool_off, int maps) {
+  // mode / pool / pool_off: see PageWalk.  maps (own only): key heads per value head
   // own: a slot's weights meet the values of its own KV head only (n_chunks chunks of VALL channels per KV head,
   // out [rows, heads, n_chunks * VALL]); else those of every KV head (n_chunks chunks over all of them)
   constexpr int KS = DIM / 32;
@@ -768,7 +860,7 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
   // a wave owns NSUB runs of 16 slots: every K and V^T fragment it reads from LDS serves all of them
   const int n_slots = n_rows * rep;
   bool valid[NSUB];
-  int head[NSUB], my_pos[NSUB];
+  int head[NSUB], my_pos[NSUB], my_blocks[NSUB];
   long row[NSUB];
 #pragma unroll
   for (int u = 0; u < NSUB; ++u) {
@@ -778,9 +870,10 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     head[u] = group * rep + (valid[u] ? slot % rep : 0);
     row[u] = row0 + tok;
     my_pos[u] = valid[u] ? pos0 + tok : -1;
+    my_blocks[u] = pool > 0 ? seen_blocks(my_pos[u], window, pool) : 0;
   }
   const bool wave_active = wave * NSUB * 16 < n_slots;  // wave-uniform
-  const PageWalk walk(pos0, pos0 + n_rows - 1, window, keep_first);
+  const PageWalk walk(pos0, pos0 + n_rows - 1, window, keep_first, mode, pool);
   const int* bt = block_tables + (long)seq * bt_stride;
   const long k_off = (long)group * DIM, k_row = (long)kv_heads * DIM, v_off = (long)PAGE * kv_heads * DIM;
 
@@ -808,7 +901,7 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
 
   u32x4 kb[KB], vb[VB];
   auto fetch = [&](int i) {
-    const uint16_t* src = cache + (long)bt[walk.page(i)] * page_stride;
+    const uint16_t* src = cache + (long)bt[walk.page(i)] * page_stride + (walk.pooled(i) ? pool_off : 0);
 #pragma unroll
     for (int b = 0; b < KB; ++b) {
       const int id = tid + 256 * b, dc = id % (DIM / 8), key = id / (DIM / 8);
@@ -816,7 +909,7 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     }
 #pragma unroll
     for (int b = 0; b < VB; ++b)
-      vb[b] = *reinterpret_cast<const u32x4*>(src + v_off + (long)(own ? group * n_chunks + chunk : chunk) * VALL * PAGE +
+      vb[b] = *reinterpret_cast<const u32x4*>(src + v_off + (long)(own ? group / maps * n_chunks + chunk : chunk) * VALL * PAGE +
                                               (long)(tid + 256 * b) * 8);
   };
   auto stash = [&]() {
@@ -845,6 +938,7 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     if (i + 1 < i_end) fetch(i + 1);
     if (!wave_active) continue;
     const int j0 = walk.page(i) * PAGE;
+    const bool pooled = walk.pooled(i);
     f32x4 s[NSUB][4];
 #pragma unroll
     for (int u = 0; u < NSUB; ++u)
@@ -870,7 +964,7 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
         for (int e = 0; e < 4; ++e) {
           const int j = j0 + 32 * (nt >> 1) + 8 * g + 4 * (nt & 1) + e;
           float v = -INFINITY;
-          if (key_seen(j, my_pos[u], window, keep_first)) {
+          if (pooled ? j < my_blocks[u] : key_seen(j, my_pos[u], window, keep_first, mode)) {
             v = s[u][nt][e] * scale;
             if (softcap > 0.f) {  // cap * tanh(v / cap), tanh(x) = 1 - 2 / (exp(2 x) + 1)
               const float x = v * inv_cap;
@@ -1058,7 +1152,10 @@ static int scan_run(const void* proj, long p_stride, int q_col, int k_col, int v
                     const int* positions, const float* decay, const float* cos_sin, int rot_dims, int layout,
                     float k_scale, const float* gate_bias, const float* gate_lower, float* out, int gated,
                     const int* pieces, const int* seq_pieces, int n_pieces, float* ws_state, float* ws_decay,
-                    float* prep, int rows, int fold, int dt, hipStream_t stream, int prepared, int vsrc, int unit_col) {
+                    float* prep, int rows, int fold, int dt, hipStream_t stream, int prepared, int vsrc, int unit_col,
+                    int act = 0) {
+  // act: 1 = q, k and v pass through silu (fixed-decay form)
+  if (act && (gated || prepared || rot_dims)) return 6;
   if (n_seqs <= 0 || rows <= 0) return 0;
   int rpt, r;
   scan_shape(dim, &rpt, &r);
@@ -1073,7 +1170,7 @@ static int scan_run(const void* proj, long p_stride, int q_col, int k_col, int v
 #define SCAN(RPT, G, F, PH, NZ)                                                                                        \
   recurrent_scan_kernel<T, RPT, G, F, PH><<<dim3(col_blocks, heads, NZ), 256, lds, stream>>>(                          \
       (const T*)proj, p_stride, v_col, heads, dim, vdim, prep, state, state_stride, seq_cu, seq_state, positions,     \
-      decay, out, r, tb, pieces, ws_state, vsrc, unit_col)
+      decay, out, r, tb, pieces, ws_state, vsrc, unit_col, act)
 #define SCAN_R(G, F, PH, NZ)                       \
   if (rpt == 8) SCAN(8, G, F, PH, NZ);             \
   else if (rpt == 16) SCAN(16, G, F, PH, NZ);      \
@@ -1086,11 +1183,11 @@ static int scan_run(const void* proj, long p_stride, int q_col, int k_col, int v
   } else if (gated) {
     SM_DISPATCH(dt, (scan_prepare_kernel<T, true><<<rows, 256, 0, stream>>>((const T*)proj, p_stride, q_col, k_col, heads,
                                                                             dim, positions, cos_sin, rot_dims, layout,
-                                                                            k_scale, gate_bias, gate_lower, prep)));
+                                                                            k_scale, gate_bias, gate_lower, prep, act)));
   } else {
     SM_DISPATCH(dt, (scan_prepare_kernel<T, false><<<rows, 256, 0, stream>>>((const T*)proj, p_stride, q_col, k_col, heads,
                                                                              dim, positions, cos_sin, rot_dims, layout,
-                                                                             k_scale, gate_bias, gate_lower, prep)));
+                                                                             k_scale, gate_bias, gate_lower, prep, act)));
   }
   if (!pieces) {
     SM_DISPATCH(dt, SCAN_G(0, n_seqs));
@@ -1122,10 +1219,10 @@ VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, 
                                     int rot_dims, int layout, float k_scale, const float* gate_bias,
                                     const float* gate_lower, float* out, int gated, const int* pieces,
                                     const int* seq_pieces, int n_pieces, float* ws_state, float* ws_decay, float* prep,
-                                    int rows, int fold, int dt, hipStream_t stream) {
+                                    int rows, int fold, int act, int dt, hipStream_t stream) {
   return scan_run(proj, p_stride, q_col, k_col, v_col, heads, dim, vdim, state, state_stride, seq_cu, seq_state, n_seqs,
                   positions, decay, cos_sin, rot_dims, layout, k_scale, gate_bias, gate_lower, out, gated, pieces,
-                  seq_pieces, n_pieces, ws_state, ws_decay, prep, rows, fold, dt, stream, 0, vdim, 0);
+                  seq_pieces, n_pieces, ws_state, ws_decay, prep, rows, fold, dt, stream, 0, vdim, 0, act);
 }
 
 // The recurrence over rows the caller prepared: prep fp32 [rows, heads, 3, dim] = q' | k' | a, values from `v`
@@ -1188,12 +1285,36 @@ VPSA_EXPORT int vpsa_head_rms(const float* o, const float* w, const void* gate, 
 // proj rows: q | k | v when own (the layer caches its keys and values), q alone otherwise.
 VPSA_EXPORT int vpsa_qk_norm_write(const void* proj, long p_stride, int heads, int kv_heads, int dim, int vdim, int own,
                                    const int* positions, const long* slots, float eps, float coef, float every,
-                                   void* q_out, void* cache, long page_stride, int rows, int dt, hipStream_t stream) {
+                                   void* q_out, void* cache, long page_stride, int rows, int v_heads, const float* qw,
+                                   const float* kw, const float* cos_sin, int rot_dims, int layout, int dt,
+                                   hipStream_t stream) {
   if (rows <= 0) return 0;
   if (coef != 0.f && !(every > 0.f)) return 2;
-  SM_DISPATCH(dt, (qk_norm_write_kernel<T><<<rows, 256, 0, stream>>>((const T*)proj, p_stride, heads, kv_heads, dim, vdim,
-                                                                     own, positions, slots, eps, coef, every, (T*)q_out,
-                                                                     (T*)cache, page_stride)));
+  if (rot_dims < 0 || rot_dims > dim || rot_dims % 2 || (rot_dims && !cos_sin) || v_heads < 1) return 3;
+  SM_DISPATCH(dt, (qk_norm_write_kernel<T><<<rows, 256, 0, stream>>>(
+                      (const T*)proj, p_stride, heads, kv_heads, dim, vdim, own, positions, slots, eps, coef, every,
+                      (T*)q_out, (T*)cache, page_stride, v_heads, qw, kw, rot_dims ? cos_sin : nullptr, rot_dims, layout)));
+  return 0;
+}
+
+// nk / nv: key and value channels per token of the layer's page regions (all heads)
+VPSA_EXPORT int vpsa_pool_blocks(void* cache, long page_stride, long pool_off, const int* block_tables, int bt_stride,
+                                 const int* row_seq, const int* positions, const long* slots, int rows, int nk, int nv,
+                                 int pool, int dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (pool < 1 || pool_off < (long)PAGE * (nk + nv)) return 2;
+  SM_DISPATCH(dt, (pool_blocks_kernel<T><<<rows, 256, 0, stream>>>((T*)cache, page_stride, pool_off, block_tables, bt_stride,
+                                                                   row_seq, positions, slots, nk, nv, pool)));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_diff_heads(const float* u, void* y, int rows, int heads, int kv_heads, int vdim, float lambda,
+                                float eps, float post, int dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (kv_heads < 1 || heads % kv_heads) return 2;
+  const long pairs = (long)rows * heads;
+  SM_DISPATCH(dt, (diff_heads_kernel<T><<<(unsigned)((pairs + 3) / 4), 256, 0, stream>>>(
+                      u, (T*)y, pairs, heads, heads / kv_heads, vdim, lambda, eps, post)));
   return 0;
 }
 
@@ -1219,14 +1340,16 @@ VPSA_EXPORT int vpsa_short_conv_qkv(const void* proj, long p_stride, const float
 VPSA_EXPORT int vpsa_window_attention(const void* q, long q_stride, const void* cache, long page_stride,
                                       const int* block_tables, int bt_stride, const int* row_seq, const int* positions,
                                       const float* sink, float* out, int rows, int heads, int kv_heads, int dim, int vdim,
-                                      int window, int keep_first, float scale, float softcap, int own, int dt,
-                                      hipStream_t stream) {
+                                      int window, int keep_first, float scale, float softcap, int own, int mode,
+                                      int pool, long pool_off, int maps, int dt, hipStream_t stream) {
   if (rows <= 0) return 0;
   if ((own ? vdim : kv_heads * vdim) > 256 * WA_ACC || (size_t)dim * 4 > 32 * 1024 || heads % kv_heads) return 2;
+  if (window < 1 || maps < 1 || kv_heads % maps || (maps > 1 && !own) || (pool > 0 && (keep_first || mode))) return 4;
   dim3 grid(rows, heads);
   SM_DISPATCH(dt, (window_attention_kernel<T><<<grid, 256, (size_t)dim * 4, stream>>>(
                       (const T*)q, q_stride, (const T*)cache, page_stride, block_tables, bt_stride, row_seq, positions,
-                      sink, out, heads, kv_heads, dim, vdim, window, keep_first, scale, softcap, own)));
+                      sink, out, heads, kv_heads, dim, vdim, window, keep_first, scale, softcap, own, mode, pool, pool_off,
+                      maps)));
   return 0;
 }
 
@@ -1251,8 +1374,8 @@ template <int DIM, int VALL, int NSUB>
 static int launch_window_mfma(const void* q, long q_stride, const void* cache, long page_stride, const int* block_tables,
                               int bt_stride, const int* tiles, const int* positions, const float* sink, float* out,
                               int n_tiles, int heads, int kv_heads, int window, int keep_first, float scale,
-                              float softcap, int splits, float* ws_o, float* ws_ml, int n_chunks, int own,
-                              hipStream_t st) {
+                              float softcap, int splits, float* ws_o, float* ws_ml, int n_chunks, int own, int mode,
+                              int pool, long pool_off, int maps, hipStream_t st) {
   constexpr int LDS = PAGE * (DIM * 2 + 16) + VALL * (PAGE * 2 + 16);
   static bool attr_set = false;
   if (!attr_set) {
@@ -1263,7 +1386,8 @@ static int launch_window_mfma(const void* q, long q_stride, const void* cache, l
   }
   window_mfma_kernel<DIM, VALL, NSUB><<<dim3(n_tiles, kv_heads * n_chunks, splits), dim3(256), LDS, st>>>(
       (const uint16_t*)q, q_stride, (const uint16_t*)cache, page_stride, block_tables, bt_stride, tiles, positions, sink,
-      out, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o, ws_ml, n_chunks, own);
+      out, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o, ws_ml, n_chunks, own, mode, pool, pool_off,
+      maps);
   if (splits > 1)  // decode rows only: row r of the launch is row r of out
     window_merge_kernel<<<n_tiles * heads, 128, 0, st>>>(ws_o, ws_ml, sink, out, heads, VALL * n_chunks, splits);
   return 0;
@@ -1278,9 +1402,10 @@ VPSA_EXPORT int vpsa_window_attention_mfma(const void* q, long q_stride, const v
                                            const int* block_tables, int bt_stride, const int* tiles,
                                            const int* positions, const float* sink, float* out, int n_tiles, int heads,
                                            int kv_heads, int dim, int vdim, int window, int keep_first, float scale,
-                                           float softcap, int splits, float* ws_o, float* ws_ml, int own,
-                                           hipStream_t stream) {
+                                           float softcap, int splits, float* ws_o, float* ws_ml, int own, int mode,
+                                           int pool, long pool_off, int maps, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
+  if (window < 1 || maps < 1 || kv_heads % maps || (maps > 1 && !own) || (pool > 0 && (keep_first || mode))) return 4;
   if (!vpsa_window_mfma_supported(heads, kv_heads, dim, vdim, own)) return 2;
   if (splits < 1 || (splits > 1 && (tiles || !ws_o || !ws_ml))) return 3;  // splits are for decode rows
   const int vall = window_chunk(own ? vdim : kv_heads * vdim), n_chunks = (own ? vdim : kv_heads * vdim) / vall;
@@ -1290,10 +1415,10 @@ VPSA_EXPORT int vpsa_window_attention_mfma(const void* q, long q_stride, const v
       return launch_window_mfma<D, V, WINDOW_PREFILL_SUB>(q, q_stride, cache, page_stride, block_tables, bt_stride,    \
                                                           tiles, positions, sink, out, n_tiles, heads, kv_heads,      \
                                                           window, keep_first, scale, softcap, splits, ws_o, ws_ml,     \
-                                                          n_chunks, own, stream);                                     \
+                                                          n_chunks, own, mode, pool, pool_off, maps, stream);         \
     return launch_window_mfma<D, V, 1>(q, q_stride, cache, page_stride, block_tables, bt_stride, tiles, positions,     \
                                        sink, out, n_tiles, heads, kv_heads, window, keep_first, scale, softcap,       \
-                                       splits, ws_o, ws_ml, n_chunks, own, stream);                                   \
+                                       splits, ws_o, ws_ml, n_chunks, own, mode, pool, pool_off, maps, stream);       \
   }
   WM(64, 128) WM(64, 256) WM(64, 512) WM(128, 128) WM(128, 256) WM(128, 512)
 #undef WM

@@ -63,6 +63,7 @@ class FeedForwardSpec:
     groups: int = 1
     keep: int = 1
     route_scale: float = 1.0
+    norm_topk: bool = False    # sigmoid router: the chosen scores are divided by their sum (+ 1e-20) first
     limit: float = 0.0
     shared_ff: int = 0
     shared_limit: float = 0.0
@@ -86,8 +87,11 @@ class RotarySpec:
     dims: int
     layout: str = "half"
     scaling: tuple | None = None
+    linear: float | None = None   # every frequency divided by this factor (position interpolation)
 
     def table_scaling(self) -> dict | None:
+        if self.linear is not None:
+            return {"rope_type": "linear", "factor": self.linear}
         if self.scaling is None:
             return None
         factor, original, fast, slow = self.scaling
@@ -167,14 +171,86 @@ class GatedRecurrenceSpec:
 
 @dataclass(frozen=True)
 class ParallelMixerSpec:
-    """Two mixers that read the same input; the layer adds left_scale * left + right_scale * right."""
-    left: WindowAttentionSpec
-    right: GatedRecurrenceSpec
+    """Two mixers that read the same input; the layer adds left_scale * left + right_scale * right.  ``normed``:
+    each output is first RMS-normed over the model width with a weight vector of its own."""
+    left: object
+    right: object
     left_scale: float
     right_scale: float
+    normed: bool = False
 
     def weight_count(self, width: int) -> int:
         return self.left.weight_count(width) + self.right.weight_count(width)
+
+
+@dataclass(frozen=True)
+class DiffAttentionSpec:
+    """Differential grouped-query attention: every head has two query / key maps over the same values,
+    o = a1 - lambda a2 with one learned lambda per layer (exp(lq1 . lk1) - exp(lq2 . lk2) + ``diff``), brought to
+    unit RMS per head and multiplied by 1 - ``diff``.  q and k are RMS-normed per head and map (one weight vector
+    each), rotary positions on their first ``rot.dims`` channels; ``chunk`` > 0: a position sees the keys of its own
+    chunk of that many positions (counted from 0) up to itself, 0: plain causal."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    diff: float
+    rot: RotarySpec
+    chunk: int
+    scale: float
+
+    def cache_elems(self) -> int:        # per token: both key maps and the values of every KV head
+        return self.kv_heads * (2 * self.dim + self.vdim)
+
+    def weight_count(self, width: int) -> int:
+        return width * (2 * self.heads * self.dim + self.kv_heads * (2 * self.dim + self.vdim)) + self.heads * self.vdim * width
+
+    def token_flops(self) -> float:      # a bound: both maps over a full chunk (a quarter of a 32k context without one)
+        return 4.0 * self.heads * (self.dim + self.vdim) * (self.chunk or 8192)
+
+
+@dataclass(frozen=True)
+class PooledWindowSpec:
+    """Grouped-query softmax attention over a sliding window of ``window`` positions and, in the same softmax, one
+    mean key / mean value per block of ``pool`` tokens that lies wholly before the window (0: none).  q and k are
+    RMS-normed per head (one weight vector each), rotary positions on their first ``rot.dims`` channels."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    window: int
+    pool: int
+    rot: RotarySpec
+    scale: float
+
+    def cache_elems(self) -> int:        # per token: keys and values, and as much again for the pooled entries
+        return self.kv_heads * (self.dim + self.vdim) * (2 if self.pool else 1)
+
+    def weight_count(self, width: int) -> int:
+        return width * (self.heads * self.dim + self.kv_heads * (self.dim + self.vdim)) + self.heads * self.vdim * width
+
+    def token_flops(self) -> float:      # the window, and the blocks of a context of 16 windows
+        keys = min(self.window, 32768) * (1 + (16 // self.pool if self.pool else 0))
+        return 2.0 * self.heads * (self.dim + self.vdim) * keys
+
+
+@dataclass(frozen=True)
+class LightningSpec:
+    """Linear attention with one fixed decay per head on silu'd projections: S <- decay S + k v^T, o = S^T q with
+    q, k, v = silu(W h); the heads side by side are RMS-normed together (one weight vector), gated by sigmoid(W_g h)."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+
+    def state_elems(self) -> int:
+        return self.heads * self.dim * self.vdim
+
+    def weight_count(self, width: int) -> int:
+        return width * self.heads * (2 * self.dim + 2 * self.vdim) + self.heads * self.vdim * width
+
+    def token_flops(self) -> float:
+        return 4.0 * self.heads * self.dim * self.vdim
 
 
 @dataclass(frozen=True)
@@ -304,6 +380,89 @@ def pelatar_config(name: str, vocab: int, width: int, layers: list[dict], norm_e
         bos_token_id=0, eos_token_id=-1)  # the design names no special tokens
 
 
+def _positive(i: int, **values) -> None:
+    for k, v in values.items():
+        if v < 1:
+            raise ValueError(f"layer {i}: {k} must be at least 1")
+
+
+def zetalorn_layers(layers: list[dict]) -> tuple:
+    """The ``layers`` list of a Zetalorn config.json -> layer specs."""
+
+    def rotary(rot: dict | None, layout: str, dim: int, i: int) -> RotarySpec:
+        rot = rot or {"base": 10000.0, "dims": 0}
+        sc = rot.get("scaling")
+        spec = RotarySpec(float(rot["base"]), int(rot["dims"]), layout, None, float(sc["factor"]) if sc else None)
+        if spec.dims % 2 or not 0 <= spec.dims <= dim or (spec.linear is not None and spec.linear <= 0):
+            raise ValueError(f"layer {i}: rotary dims must be even and within the head, a scaling factor positive")
+        return spec
+
+    out = []
+    for i, entry in enumerate(layers):
+        m = entry["mixer"]
+        kind = entry["type"]
+        if kind == "attention":
+            mask = m.get("mask") or {}
+            mixer = DiffAttentionSpec(
+                heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                diff=float(m["diff"]), rot=rotary(m.get("rot"), "pairs", int(m["dim"]), i), chunk=int(mask.get("size", 0)),
+                scale=float(m["scale"]))
+            _positive(i, heads=mixer.heads, kv_heads=mixer.kv_heads, dim=mixer.dim, vdim=mixer.vdim)
+            if mixer.heads % mixer.kv_heads or mixer.chunk < 0:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads and the chunk size positive")
+        elif kind == "parallel":
+            a, r = m["left"], m["right"]
+            mask = a.get("mask") or {}
+            left = PooledWindowSpec(
+                heads=int(a["heads"]), kv_heads=int(a["kv_heads"]), dim=int(a["dim"]), vdim=int(a["vdim"]),
+                window=int(mask.get("size", 1 << 30)), pool=int(mask.get("pool", 0)),
+                rot=rotary(a.get("rot"), "half", int(a["dim"]), i), scale=float(a["scale"]))
+            _positive(i, heads=left.heads, kv_heads=left.kv_heads, dim=left.dim, vdim=left.vdim, window=left.window)
+            if left.heads % left.kv_heads or left.pool < 0:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads and the pooled block size positive")
+            right = LightningSpec(int(r["heads"]), int(r["dim"]), int(r["vdim"]), tuple(float(d) for d in r["decay"]))
+            _positive(i, right_heads=right.heads, right_dim=right.dim, right_vdim=right.vdim)
+            if len(right.decay) != right.heads or not all(0.0 <= d <= 1.0 for d in right.decay):
+                raise ValueError(f"layer {i}: one decay within [0, 1] per head is required")
+            mixer = ParallelMixerSpec(left, right, 0.5, 0.5, normed=True)
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        f = entry.get("mlp")
+        mlp = None
+        if f is not None:
+            if f.get("kind", "moe") != "moe":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+            r, ex = f["router"], f["expert"]
+            g = r.get("groups") or {}
+            mlp = FeedForwardSpec(
+                kind="moe", ff=int(ex["ff"]), gated=True, experts=int(r["experts"]), top=int(r["top"]),
+                groups=int(g.get("count", 1)), keep=int(g.get("keep", g.get("count", 1))), norm_topk=True,
+                limit=float(ex["limit"]))
+            if (mlp.groups < 1 or mlp.experts % mlp.groups or not 1 <= mlp.keep <= mlp.groups
+                    or not 1 <= mlp.top <= mlp.experts // mlp.groups * mlp.keep or mlp.ff < 1):
+                raise ValueError(f"layer {i}: experts must split into equal groups, and the kept groups hold `top`")
+        out.append(LayerSpec(kind, mixer, mlp))
+    return tuple(out)
+
+
+def zetalorn_config(name: str, vocab: int, width: int, layers: list[dict], loop: dict | None = None,
+                    logit_scale: float = 1.0, norm_eps: float = 1e-6, max_position_embeddings: int = 32768) -> "ModelConfig":
+    specs = zetalorn_layers(layers)
+    runs = None
+    if loop:
+        runs = (int(loop["start"]), int(loop["stop"]), int(loop["times"]))
+        if not 0 <= runs[0] < runs[1] <= len(specs) or runs[2] < 1:
+            raise ValueError("loop: 0 <= start < stop <= layers and times >= 1 are required")
+    att = [s.mixer.left if s.type == "parallel" else s.mixer for s in specs]
+    return ModelConfig(
+        name=name, architecture="zetalorn", vocab_size=int(vocab), hidden_size=int(width),
+        intermediate_size=max([s.mlp.ff for s in specs if s.mlp] + [0]), num_layers=len(specs),
+        num_heads=max(a.heads for a in att), num_kv_heads=max(a.kv_heads for a in att),
+        head_dim=max(a.dim for a in att), norm_eps=float(norm_eps), max_position_embeddings=max_position_embeddings,
+        tie_word_embeddings=False, logit_scale=float(logit_scale), layer_specs=specs, layer_loop=runs,
+        bos_token_id=0, eos_token_id=-1)  # the design names no special tokens
+
+
 def _rotary(rot: dict, layout: str) -> RotarySpec:
     sc = rot.get("scaling")
     scaling = None if not sc else (float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"]))
@@ -415,7 +574,7 @@ def zururax_config(name: str, vocab: int, width: int, layers: list[dict], embedd
 @dataclass
 class ModelConfig:
     name: str = "tiny-llama"
-    architecture: str = "llama"  # llama | mixtral | opt | gpt2 | zururax | revelix | pelatar
+    architecture: str = "llama"  # llama | mixtral | opt | gpt2 | zururax | revelix | pelatar | zetalorn
     vocab_size: int = 512
     hidden_size: int = 256
     intermediate_size: int = 512
@@ -442,6 +601,20 @@ class ModelConfig:
     layer_specs: tuple = ()
     embedding_scale: float = 1.0
     logit_scale: float = 1.0   # logits = head(x) * logit_scale
+    # (start, stop, times): layers start .. stop - 1 run `times` times in a row with the same weights, every pass
+    # with cache entries and state of its own
+    layer_loop: tuple | None = None
+
+    def layer_runs(self) -> list:
+        """(layer index, pass number when the run starts a pass of the loop, else None) of every layer run."""
+        n = len(self.layer_specs)
+        if not self.layer_loop:
+            return [(i, None) for i in range(n)]
+        start, stop, times = self.layer_loop
+        runs = [(i, None) for i in range(start)]
+        for t in range(times):
+            runs += [(i, t if i == start else None) for i in range(start, stop)]
+        return runs + [(i, None) for i in range(stop, n)]
 
     @property
     def q_size(self) -> int:
@@ -456,7 +629,7 @@ class ModelConfig:
         h, i = self.hidden_size, self.intermediate_size
         if self.layer_specs:
             gemm = pair = 0.0
-            for s in self.layer_specs:
+            for s in [self.layer_specs[i] for i, _ in self.layer_runs()]:
                 m, f = s.mixer, s.mlp
                 gemm += m.weight_count(h)
                 if isinstance(m, LatentMixerSpec):
@@ -721,6 +894,10 @@ def _from_hf_config(cfg: dict[str, Any], name: str) -> ModelConfig:
         return revelix_config(name, cfg["vocab"], cfg["width"], cfg["layers"], logit_scale=cfg.get("logit_scale", 1.0),
                               norm_eps=(cfg.get("norm") or {}).get("eps", 1e-6),
                               max_position_embeddings=int(cfg.get("max_positions", 32768)))
+    if str(cfg.get("architecture", "")).lower() == "zetalorn":
+        return zetalorn_config(name, cfg["vocab"], cfg["width"], cfg["layers"], loop=cfg.get("loop"),
+                               logit_scale=cfg.get("logit_scale", 1.0), norm_eps=(cfg.get("norm") or {}).get("eps", 1e-6),
+                               max_position_embeddings=int(cfg.get("max_positions", 32768)))
     if str(cfg.get("architecture", "")).lower() == "pelatar":
         return pelatar_config(name, cfg["vocab"], cfg["width"], cfg["layers"],
                               norm_eps=(cfg.get("norm") or {}).get("eps", 1e-5),

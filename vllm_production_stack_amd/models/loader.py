@@ -19,6 +19,7 @@ from .opt import OPTModel
 from .transformer import LayerWeights, TransformerModel
 from .pelatar import PelatarModel
 from .revelix import RevelixModel
+from .zetalorn import ZetalornModel
 from .zururax import ZururaxModel
 
 
@@ -33,6 +34,8 @@ def build_model(cfg: ModelConfig, dtype: torch.dtype, device: torch.device, max_
         model = RevelixModel(cfg, dtype, device, max_model_len)
     elif cfg.architecture == "pelatar":
         model = PelatarModel(cfg, dtype, device, max_model_len)
+    elif cfg.architecture == "zetalorn":
+        model = ZetalornModel(cfg, dtype, device, max_model_len)
     else:
         model = TransformerModel(cfg, dtype, device, max_model_len, expert_parallel=expert_parallel)
     has_weights = ckpt_dir is not None and any(Path(ckpt_dir).glob("*.safetensors"))
@@ -68,6 +71,8 @@ def load_hf_weights(model, ckpt_dir: Path) -> None:
         _load_revelix(model, ckpt_dir)
     elif isinstance(model, PelatarModel):
         _load_pelatar(model, ckpt_dir)
+    elif isinstance(model, ZetalornModel):
+        _load_zetalorn(model, ckpt_dir)
     else:
         _load_llama(model, ckpt_dir)
 
@@ -585,5 +590,124 @@ def _load_pelatar(model: PelatarModel, ckpt_dir: Path) -> None:
             else:
                 want |= {f"l{i}.mlp.router", f"l{i}.mlp.correction"}
                 want |= {f"l{i}.mlp.e{e}.{k}" for e in range(f.experts) for k in ("gate", "up", "down")}
+    if want - seen:
+        raise ValueError(f"checkpoint lacks {sorted(want - seen)[:8]}")
+
+
+def _load_zetalorn(model: ZetalornModel, ckpt_dir: Path) -> None:
+    """Zetalorn checkpoints: ``embed``, ``head``, ``final.norm``, ``loop.step`` (models with a layer loop); per layer
+    ``l<i>.norm1|norm2`` (one number each), ``l<i>.rg1|rg2`` with ``.b`` (the residual gates), ``l<i>.mix.{q, k, v,
+    q.norm, k.norm, lq1, lk1, lq2, lk2, o}`` (attention) or ``l<i>.mix.left.{q, k, v, q.norm, k.norm, o, out}`` and
+    ``l<i>.mix.right.{q, k, v, g, norm, o, out}`` (parallel), ``l<i>.mlp.router`` and ``l<i>.mlp.e<j>.{gate, up, down}``.
+    Linear weights are [out, in]; a mixer's input projections and the mixer's residual gate are fused row-wise
+    here, the units stacked, the norms' single numbers spread over the width.  The query rows of a differential
+    attention (stored head by head as map 1 | map 2) are reordered to group, map, head in group.  Every tensor
+    the model holds must be found, and every tensor of the file must have a place."""
+    from ..engine.config import DiffAttentionSpec
+
+    pat = re.compile(r"l(\d+)\.(.+)")
+    unit = re.compile(r"mlp\.e(\d+)\.(gate|up|down)")
+    seen: set[str] = set()
+
+    def put(dst: torch.Tensor, src: torch.Tensor, what: str) -> None:
+        if tuple(dst.shape) != tuple(src.shape):
+            raise ValueError(f"{what}: checkpoint shape {tuple(src.shape)}, model expects {tuple(dst.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+    def put_scalar(dst: torch.Tensor, src: torch.Tensor, what: str) -> None:
+        if src.numel() != 1:
+            raise ValueError(f"{what}: one number expected, checkpoint shape {tuple(src.shape)}")
+        dst.fill_(float(src.float().reshape(())))
+
+    for name, t in _iter_safetensors(ckpt_dir):
+        seen.add(name)
+        if name == "embed":
+            put(model.embed, t, name)
+            continue
+        if name == "head":
+            put(model.lm_head, t, name)
+            continue
+        if name == "final.norm":
+            put_scalar(model.norm, t, name)
+            continue
+        if name == "loop.step" and model.loop_step is not None:
+            put(model.loop_step, t, name)
+            continue
+        mt = pat.match(name)
+        if not mt or int(mt.group(1)) >= len(model.layers):
+            raise ValueError(f"unexpected tensor {name!r}")
+        lw = model.layers[int(mt.group(1))]
+        sub = mt.group(2)
+        m, f = lw.spec.mixer, lw.spec.mlp
+        rows = model.in_rows(lw.spec)
+        diff = isinstance(m, DiffAttentionSpec)
+        ok = True
+        um = unit.fullmatch(sub)
+        if sub == "norm1":
+            put_scalar(lw.norm1, t, name)
+        elif sub == "rg1":
+            put(lw.w_in[rows["rg1"][0]:rows["rg1"][1]], t, name)
+        elif sub == "rg1.b":
+            put(lw.rg1_b, t, name)
+        elif f is not None and sub == "norm2":
+            put_scalar(lw.norm2, t, name)
+        elif f is not None and sub == "rg2":
+            put(lw.rg2, t, name)
+        elif f is not None and sub == "rg2.b":
+            put(lw.rg2_b, t, name)
+        elif f is not None and sub == "mlp.router":
+            put(lw.router, t, name)
+        elif f is not None and um and int(um.group(1)) < f.experts:
+            e, which = int(um.group(1)), um.group(2)
+            if which == "down":
+                put(lw.w2[e], t, name)
+            else:
+                put(lw.w13[e, :f.ff] if which == "gate" else lw.w13[e, f.ff:], t, name)
+        elif diff and sub == "mix.q":
+            a, b = rows["q"]
+            if tuple(t.shape) != (b - a, lw.w_in.shape[1]):
+                raise ValueError(f"{name}: checkpoint shape {tuple(t.shape)}, model expects {(b - a, lw.w_in.shape[1])}")
+            rep = m.heads // m.kv_heads
+            t = t.view(m.kv_heads, rep, 2, m.dim, -1).permute(0, 2, 1, 3, 4).reshape(b - a, -1)
+            put(lw.w_in[a:b], t, name)
+        elif diff and sub in ("mix.k", "mix.v"):
+            a, b = rows[sub[4:]]
+            put(lw.w_in[a:b], t, name)
+        elif diff and sub in ("mix.lq1", "mix.lk1", "mix.lq2", "mix.lk2"):
+            put(lw.lam_vecs[("lq1", "lk1", "lq2", "lk2").index(sub[4:])], t, name)
+        elif not diff and sub.startswith("mix.") and sub[4:] in rows and sub[4:] != "rg1":
+            a, b = rows[sub[4:]]
+            put(lw.w_in[a:b], t, name)
+        elif sub in ("mix.q.norm", "mix.left.q.norm") and diff == (sub == "mix.q.norm"):
+            put(lw.q_norm, t, name)
+        elif sub in ("mix.k.norm", "mix.left.k.norm") and diff == (sub == "mix.k.norm"):
+            put(lw.k_norm, t, name)
+        elif sub in ("mix.o", "mix.left.o") and diff == (sub == "mix.o"):
+            put(lw.w_o, t, name)
+        elif not diff and sub == "mix.right.o":
+            put(lw.wr_o, t, name)
+        elif not diff and sub == "mix.right.norm":
+            put(lw.r_norm, t, name)
+        elif not diff and sub == "mix.left.out":
+            put(lw.left_out, t, name)
+        elif not diff and sub == "mix.right.out":
+            put(lw.right_out, t, name)
+        else:
+            ok = False
+        if not ok:
+            raise ValueError(f"unexpected tensor {name!r}")
+    want = {"embed", "head", "final.norm"} | ({"loop.step"} if model.loop_step is not None else set())
+    for i, lw in enumerate(model.layers):
+        m, f = lw.spec.mixer, lw.spec.mlp
+        want |= {f"l{i}.{k}" for k in ("norm1", "rg1", "rg1.b")}
+        if isinstance(m, DiffAttentionSpec):
+            want |= {f"l{i}.mix.{k}" for k in ("q", "k", "v", "q.norm", "k.norm", "lq1", "lk1", "lq2", "lk2", "o")}
+            model.set_lambda(lw)
+        else:
+            want |= {f"l{i}.mix.left.{k}" for k in ("q", "k", "v", "q.norm", "k.norm", "o", "out")}
+            want |= {f"l{i}.mix.right.{k}" for k in ("q", "k", "v", "g", "norm", "o", "out")}
+        if f is not None:
+            want |= {f"l{i}.{k}" for k in ("norm2", "rg2", "rg2.b", "mlp.router")}
+            want |= {f"l{i}.mlp.e{e}.{k}" for e in range(f.experts) for k in ("gate", "up", "down")}
     if want - seen:
         raise ValueError(f"checkpoint lacks {sorted(want - seen)[:8]}")

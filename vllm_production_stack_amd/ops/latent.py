@@ -78,6 +78,42 @@ def add_rms_norm(residual, delta, weight, eps: float, out_dtype, want_out: bool 
     return y
 
 
+def gated_add_rms_norm(residual, deltas, gate, gate_bias, weight, eps: float, out_dtype, *, extra=None, extra_vec=None,
+                       want_out: bool = True):
+    """A gated residual in front of a pre-norm.  residual (fp32, in place) +=
+    sigmoid(gate + gate_bias) * sum_i c_i n_i(d_i) + extra + extra_vec over ``deltas``, up to two (tensor, norm weight
+    or None, factor) triples: n(d) = rmsnorm(d) * norm weight where one is given, d itself otherwise.  The first
+    delta is in the activation dtype or fp32 (a mixture's sum), the second in the activation dtype; ``gate`` is a
+    [T, n] view (of a wider projection, say) in the activation dtype or None (no gate), ``gate_bias`` fp32 [n] or
+    None; ``extra`` fp32 [T, n] (a stream that re-enters) and ``extra_vec`` fp32 [n] are added ungated.
+    Returns rmsnorm(residual) * weight in ``out_dtype`` (None without ``want_out``)."""
+    deltas = list(deltas)
+    assert len(deltas) <= 2
+    if not residual.is_cuda:
+        return reference.gated_add_rms_norm(residual, deltas, gate, gate_bias, extra, extra_vec, weight, eps, out_dtype,
+                                            want_out)
+    o = _ops()
+    _f32(residual, weight, gate_bias, extra, extra_vec)
+    t, n = residual.shape
+    if t == 0:
+        return torch.empty((0, n), dtype=out_dtype, device=residual.device) if want_out else None
+    ds = deltas + [(None, None, 0.0)] * (2 - len(deltas))
+    (d1, w1, c1), (d2, w2, c2) = ds
+    _f32(w1, w2)
+    assert d1 is None or (_rows(d1) and d1.shape == (t, n) and d1.dtype in (out_dtype, torch.float32))
+    assert d2 is None or (_rows(d2) and d2.shape == (t, n) and d2.dtype == out_dtype)
+    assert gate is None or (_rows(gate) and gate.shape == (t, n) and gate.dtype == out_dtype)
+    assert extra is None or (extra.is_contiguous() and extra.shape == (t, n))
+    y = torch.empty((t, n), dtype=out_dtype, device=residual.device) if want_out else None
+    o._check(o._kernels().vpsa_gated_add_rmsnorm(
+        o._p(residual), o._p(d1), c_long(d1.stride(0) if d1 is not None else 0),
+        c_int(1 if (d1 is not None and d1.dtype == torch.float32) else 0), o._p(w1), c_float(c1), o._p(d2),
+        c_long(d2.stride(0) if d2 is not None else 0), o._p(w2), c_float(c2), o._p(gate),
+        c_long(gate.stride(0) if gate is not None else 0), o._p(gate_bias), o._p(extra), o._p(extra_vec), o._p(weight),
+        o._p(y), c_int(t), c_int(n), c_float(eps), c_int(_DT[out_dtype]), o._stream()), "gated_add_rms_norm")
+    return y
+
+
 def rms_norm_add(residual, delta, weight, eps: float, out_dtype, want_out: bool = True):
     """A norm on a sublayer's output: residual (fp32, in place) += rmsnorm(delta) * weight.  ``delta`` is in
     ``out_dtype`` or fp32 (a mixture's sum).  Returns the new residual rounded to ``out_dtype``: the next
@@ -335,15 +371,16 @@ def route_softmax(logits, n: int, experts: int, groups: int, keep: int, topk: in
     return w, ids, gate
 
 
-def group_topk(logits, experts: int, groups: int, keep: int, topk: int, route_scale: float, extra: bool = False):
+def group_topk(logits, experts: int, groups: int, keep: int, topk: int, route_scale: float, extra: bool = False,
+               normalize: bool = False):
     """Router logits fp32 [T, >= experts (+1)] -> (weights fp32 [T, topk], ids int32 [T, topk], extra).
 
     Scores are sigmoids; experts form ``groups`` equal runs of neighbours, a group scores the sum of
     its two largest scores, and only experts of the ``keep`` best groups can be chosen; weights are
-    the chosen scores times ``route_scale``.  ``extra``: column ``experts`` is one more logit per
+    the chosen scores (``normalize``: divided by their sum + 1e-20) times ``route_scale``.  ``extra``: column ``experts`` is one more logit per
     token, returned as its sigmoid (a shared unit's gate)."""
     if not logits.is_cuda:
-        return reference.group_topk(logits, experts, groups, keep, topk, route_scale, extra)
+        return reference.group_topk(logits, experts, groups, keep, topk, route_scale, extra, normalize)
     o = _ops()
     _f32(logits)
     t = logits.shape[0]
@@ -352,7 +389,7 @@ def group_topk(logits, experts: int, groups: int, keep: int, topk: int, route_sc
     ex = torch.empty((t,), dtype=torch.float32, device=logits.device) if extra else None
     o._check(o._kernels().vpsa_group_topk(o._p(logits), c_int(logits.shape[1]), o._p(w), o._p(ids), o._p(ex), c_int(t),
                                           c_int(experts), c_int(groups), c_int(keep), c_int(topk),
-                                          c_float(route_scale), o._stream()), "group_topk")
+                                          c_float(route_scale), c_int(1 if normalize else 0), o._stream()), "group_topk")
     return w, ids, ex
 
 

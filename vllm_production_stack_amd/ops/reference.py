@@ -51,6 +51,8 @@ def build_cos_sin(head_dim: int, max_pos: int, theta: float, scaling: dict | Non
         mid = (1 - smooth) * inv / factor + smooth * inv
         is_mid = (wavelen <= orig / lo) & (wavelen >= orig / hi)
         inv = torch.where(is_mid, mid, scaled)
+    if scaling and scaling.get("rope_type", scaling.get("type")) == "linear":
+        inv = inv / float(scaling["factor"])  # position interpolation: every frequency divided by the factor
     mag = 1.0
     if scaling and scaling.get("rope_type", scaling.get("type")) == "ramp":
         # frequencies divided by ``factor`` behind a linear ramp over the pair index, between the pairs
@@ -360,6 +362,26 @@ def add_rms_norm(residual, delta, weight, eps, out_dtype, want_out=True):
     return (residual * inv * weight).to(out_dtype)
 
 
+def gated_add_rms_norm(residual, deltas, gate, gate_bias, extra, extra_vec, weight, eps, out_dtype, want_out=True):
+    total = None
+    for d, w, c in deltas:
+        d = d.float()
+        if w is not None:
+            d = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w
+        total = d * c if total is None else total + d * c
+    if total is not None:
+        if gate is not None:
+            total = total * torch.sigmoid(gate.float() + (gate_bias if gate_bias is not None else 0.0))
+        residual.add_(total)
+    if extra is not None:
+        residual.add_(extra)
+    if extra_vec is not None:
+        residual.add_(extra_vec)
+    if not want_out:
+        return None
+    return (residual * torch.rsqrt(residual.pow(2).mean(-1, keepdim=True) + eps) * weight).to(out_dtype)
+
+
 def rms_norm_add(residual, delta, weight, eps, out_dtype, want_out=True):
     d = delta.float()
     residual.add_(d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * weight)
@@ -473,7 +495,7 @@ def glu_clamp(x, limit, alpha, up_bias):
     return (g * torch.sigmoid(alpha * g) * (u + up_bias)).to(x.dtype)
 
 
-def group_topk(logits, experts, groups, keep, topk, route_scale, extra):
+def group_topk(logits, experts, groups, keep, topk, route_scale, extra, normalize=False):
     t = logits.shape[0]
     s = torch.sigmoid(logits[:, :experts].float())
     per = experts // groups
@@ -485,7 +507,10 @@ def group_topk(logits, experts, groups, keep, topk, route_scale, extra):
     allowed.scatter_(1, order, True)
     masked = torch.where(allowed[:, :, None].expand(t, groups, per).reshape(t, experts), s, torch.full_like(s, -1.0))
     ids = torch.sort(masked, dim=-1, descending=True, stable=True).indices[:, :topk]
-    w = s.gather(1, ids) * route_scale
+    w = s.gather(1, ids)
+    if normalize:
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    w = w * route_scale
     ex = torch.sigmoid(logits[:, experts].float()) if extra else None
     return w, ids.int(), ex
 
@@ -529,7 +554,7 @@ def _rotate_rows(x, pos, cos_sin, dims, layout):
 
 
 def recurrent_scan(proj, q_col, k_col, v_col, heads, dim, vdim, gated, state, state_off, seq_cu, seq_state, positions,
-                   decay, cos_sin, rot_dims, layout, k_scale, gate_bias, gate_lower):
+                   decay, cos_sin, rot_dims, layout, k_scale, gate_bias, gate_lower, act=False):
     t = proj.shape[0]
     out = torch.zeros((t, heads, vdim), dtype=torch.float32)
     q = proj[:, q_col:q_col + heads * dim].float().view(t, heads, dim)
@@ -541,6 +566,8 @@ def recurrent_scan(proj, q_col, k_col, v_col, heads, dim, vdim, gated, state, st
         a = lower + (1 - lower) * torch.sigmoid(k + gate_bias.view(1, heads, dim))
         k = 1 - a
     else:
+        if act:
+            q, k, v = (torch.nn.functional.silu(x) for x in (q, k, v))
         q = _rotate_rows(q, positions, cos_sin, rot_dims, layout)
         k = _rotate_rows(k, positions, cos_sin, rot_dims, layout) * k_scale
         a = decay.view(1, heads, 1).expand(t, heads, dim)
@@ -631,21 +658,26 @@ def head_finish(o, eps, out_dtype, vdim, stab, unit, weight, gate, gate_act):
     return y.to(out_dtype)
 
 
-def qk_norm_write(proj, heads, kv_heads, dim, vdim, positions, slots, pool, cache_off, eps, temp_coef, temp_every, own):
+def qk_norm_write(proj, heads, kv_heads, dim, vdim, positions, slots, pool, cache_off, eps, temp_coef, temp_every, own,
+                  v_heads=None, q_weight=None, k_weight=None, cos_sin=None, rot_dims=0, layout=0):
     t = proj.shape[0]
     nq, nk = heads * dim, kv_heads * dim
+    v_heads = kv_heads if v_heads is None else v_heads
 
-    def unit(x):
-        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    def unit(x, w):
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        if w is not None:
+            x = x * w
+        return _rotate_rows(x, positions, cos_sin, rot_dims, layout) if rot_dims else x
 
-    q = unit(proj[:, :nq].float().view(t, heads, dim))
+    q = unit(proj[:, :nq].float().view(t, heads, dim), q_weight)
     if temp_coef != 0.0:
         steps = torch.floor((positions.double() + 1.0) / temp_every).float()
         q = q * (1.0 + temp_coef * torch.log(steps + 1.0))[:, None, None]
     if own:
-        k = unit(proj[:, nq:nq + nk].float().view(t, kv_heads, dim)).to(pool.dtype)
-        v = proj[:, nq + nk:nq + nk + kv_heads * vdim].reshape(t, kv_heads, vdim).to(pool.dtype)
-        kc, vc = window_cache_views(pool, cache_off, kv_heads, dim, vdim)
+        k = unit(proj[:, nq:nq + nk].float().view(t, kv_heads, dim), k_weight).to(pool.dtype)
+        v = proj[:, nq + nk:nq + nk + v_heads * vdim].reshape(t, v_heads, vdim).to(pool.dtype)
+        kc, vc = window_cache_views(pool, cache_off, kv_heads, dim, vdim, v_heads)
         ok = slots >= 0
         pg, off = (slots[ok] // PAGE).long(), (slots[ok] % PAGE).long()
         kc[pg, off] = k[ok]
@@ -664,15 +696,41 @@ def head_rms_norm(o, eps, weight, gate, out_dtype):
     return y.to(out_dtype)
 
 
-def window_cache_views(pool, cache_off, kv_heads, dim, vdim):
+def window_cache_views(pool, cache_off, kv_heads, dim, vdim, v_heads=None):
     """K [pages, PAGE, kv_heads, dim] and V [pages, PAGE, kv_heads, vdim] of one layer: views of the pool
     (indexed reads and writes go through).  In a page, K is stored key by key ([PAGE][kv_heads * dim]) and V
     transposed ([kv_heads * vdim][PAGE]: a channel's 64 keys are contiguous, which is what the second matrix
     product of the attention kernels reads)."""
-    nk, nv = PAGE * kv_heads * dim, PAGE * kv_heads * vdim
+    v_heads = kv_heads if v_heads is None else v_heads  # fewer when several key maps share a value head
+    nk, nv = PAGE * kv_heads * dim, PAGE * v_heads * vdim
     k = pool[:, cache_off:cache_off + nk].view(pool.shape[0], PAGE, kv_heads, dim)
-    v = pool[:, cache_off + nk:cache_off + nk + nv].view(pool.shape[0], kv_heads, vdim, PAGE).permute(0, 3, 1, 2)
+    v = pool[:, cache_off + nk:cache_off + nk + nv].view(pool.shape[0], v_heads, vdim, PAGE).permute(0, 3, 1, 2)
     return k, v
+
+
+def pool_blocks(pool, cache_off, pool_off, kv_heads, dim, vdim, block_tables, row_seq, positions, slots, block):
+    kc, vc = window_cache_views(pool, cache_off, kv_heads, dim, vdim)
+    pk, pv = window_cache_views(pool, cache_off + pool_off, kv_heads, dim, vdim)
+    for r in range(positions.numel()):
+        p = int(positions[r])
+        if int(slots[r]) < 0 or (p + 1) % block:
+            continue
+        s = r if row_seq is None else int(row_seq[r])
+        b = p // block
+        idx = torch.arange(b * block, p + 1)
+        pages = block_tables[s].long()[idx // PAGE]
+        dst = int(block_tables[s, b // PAGE])
+        pk[dst, b % PAGE] = (kc[pages, idx % PAGE].float().sum(0) / block).to(pool.dtype)
+        pv[dst, b % PAGE] = (vc[pages, idx % PAGE].float().sum(0) / block).to(pool.dtype)
+
+
+def diff_heads(u, kv_heads, lam, eps, post, out_dtype):
+    t, h2, vdim = u.shape
+    heads = h2 // 2
+    a = u.view(t, kv_heads, 2, heads // kv_heads, vdim)
+    o = (a[:, :, 0] - lam * a[:, :, 1]).reshape(t, heads, vdim)
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * post
+    return o.reshape(t, heads * vdim).to(out_dtype)
 
 
 def short_conv_qkv(proj, conv_w, heads, kv_heads, dim, vdim, state, state_off, seq_cu, seq_state, positions, slots,
@@ -710,27 +768,38 @@ def short_conv_qkv(proj, conv_w, heads, kv_heads, dim, vdim, state, state_off, s
 
 
 def window_attention(q, pool, cache_off, kv_heads, vdim, block_tables, row_seq, positions, window, keep_first, scale,
-                     softcap, sink, out, own_values=False):
+                     softcap, sink, out, own_values=False, mode=0, pool_block=0, pool_off=0, maps=1):
     t, heads, dim = q.shape
-    kc, vc = window_cache_views(pool, cache_off, kv_heads, dim, vdim)
+    kc, vc = window_cache_views(pool, cache_off, kv_heads, dim, vdim, kv_heads // maps)
+    if pool_block:
+        pk, pv = window_cache_views(pool, cache_off + pool_off, kv_heads, dim, vdim, kv_heads // maps)
     rep = heads // kv_heads
     for r in range(t):
         s = r if row_seq is None else int(row_seq[r])
         p = int(positions[r])
-        lo = max(0, p - window + 1)
+        lo = p - p % window if mode == 1 else max(0, p - window + 1)
         keys = list(range(min(keep_first, lo))) + list(range(lo, p + 1))
         idx = torch.tensor(keys)
         pages = block_tables[s].long()[idx // PAGE]
         kk = kc[pages, idx % PAGE].float()       # [keys, kv_heads, dim]
-        vv = vc[pages, idx % PAGE].float()       # [keys, kv_heads, vdim]
+        vv = vc[pages, idx % PAGE].float()       # [keys, value heads, vdim]
+        nb = max(0, (p - window + 1) // pool_block) if pool_block else 0
+        if nb:  # one pooled entry per block of tokens that lies wholly before the window
+            idx = torch.arange(nb)
+            pages = block_tables[s].long()[idx // PAGE]
+            kk = torch.cat([pk[pages, idx % PAGE].float(), kk])
+            vv = torch.cat([pv[pages, idx % PAGE].float(), vv])
         sc = torch.einsum("hd,khd->hk", q[r].float(), kk.repeat_interleave(rep, dim=1)) * scale
         if softcap > 0:
             sc = softcap * torch.tanh(sc / softcap)
-        mx = torch.maximum(sc.max(-1).values, sink)
-        e = torch.exp(sc - mx[:, None])
-        w = e / (e.sum(-1) + torch.exp(sink - mx))[:, None]
+        if sink is None:
+            w = torch.softmax(sc, dim=-1)
+        else:
+            mx = torch.maximum(sc.max(-1).values, sink)
+            e = torch.exp(sc - mx[:, None])
+            w = e / (e.sum(-1) + torch.exp(sink - mx))[:, None]
         if own_values:
-            out[r, :, 0] = torch.einsum("hk,khv->hv", w, vv.repeat_interleave(rep, dim=1))
+            out[r, :, 0] = torch.einsum("hk,khv->hv", w, vv.repeat_interleave(rep * maps, dim=1))
         else:
             out[r] = torch.einsum("hk,kgv->hgv", w, vv)
     return out

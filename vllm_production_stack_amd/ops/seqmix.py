@@ -120,7 +120,8 @@ def build_scan_pieces(q_lens, target: int = SCAN_PIECES_TARGET):
 
 def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: int, vdim: int, state, state_off: int,
                    seq_cu, seq_state, positions, *, decay=None, cos_sin=None, rot_dims: int = 0, layout: int = 0,
-                   k_scale: float = 1.0, gate_bias=None, gate_lower=None, pieces=None, min_decay: float = 0.0):
+                   k_scale: float = 1.0, gate_bias=None, gate_lower=None, pieces=None, min_decay: float = 0.0,
+                   act: bool = False):
     """Per sequence and head, over the sequence's rows in order: S <- a_t (.) S + k_t v_t^T, o_t = S^T q_t
     with S [dim, vdim] carried in the sequence's state slot.  q, k and v are column ranges of ``proj``
     [T, cols] (heads side by side).
@@ -132,6 +133,8 @@ def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: in
     ``min_decay``: the smallest of the decays as the host knows it; from ``SCAN_FOLD_MIN_DECAY`` up the kernel
     folds the decay into the staged keys and queries of a 16-token block (two operations per state element and
     token instead of three).
+
+    ``act`` (with ``decay``, no rotation): q, k and v pass through silu first.
 
     ``gate_bias`` / ``gate_lower`` (fp32 [heads * dim]) instead: the k columns hold gate logits,
     a_t = lower + (1 - lower) sigmoid(logit + bias) per row of S, k_t = 1 - a_t, q = silu(q).
@@ -145,14 +148,14 @@ def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: in
     if not proj.is_cuda:
         return reference.recurrent_scan(proj, q_col, k_col, v_col, heads, dim, vdim, gated, state, state_off, seq_cu,
                                         seq_state, positions, decay, cos_sin, rot_dims, layout, k_scale, gate_bias,
-                                        gate_lower)
+                                        gate_lower, act)
     o = _ops()
     _f32(state, decay, cos_sin, gate_bias, gate_lower)
     _i32(seq_cu, seq_state, positions)
     assert _rows(proj) and max(q_col, k_col) + heads * dim <= proj.shape[1] and v_col + heads * vdim <= proj.shape[1]
     assert state_off + heads * dim * vdim <= state.shape[1] and seq_cu.numel() == seq_state.numel() + 1
     assert (gate_bias is not None and gate_lower is not None) if gated else (rot_dims == 0 or cos_sin.shape[1] == rot_dims)
-    assert rot_dims <= dim and rot_dims % 2 == 0
+    assert rot_dims <= dim and rot_dims % 2 == 0 and not (act and (gated or rot_dims))
     out = torch.empty((proj.shape[0], heads, vdim), dtype=torch.float32, device=proj.device)
     # what enters the recurrence besides v, prepared in fp32 by a pass of its own: q' | k' (| gates)
     prep = torch.empty((proj.shape[0], heads, 3 if gated else 2, dim), dtype=torch.float32, device=proj.device)
@@ -171,7 +174,7 @@ def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: in
         c_int(seq_state.numel()), o._p(positions), o._p(decay), o._p(cos_sin), c_int(rot_dims), c_int(layout),
         c_float(k_scale), o._p(gate_bias), o._p(gate_lower), o._p(out), c_int(1 if gated else 0), o._p(pc), o._p(sp),
         c_int(n_pieces), o._p(ws_state), o._p(ws_decay), o._p(prep), c_int(proj.shape[0]),
-        c_int(1 if (not gated and min_decay >= SCAN_FOLD_MIN_DECAY) else 0), c_int(_dt(proj)),
+        c_int(1 if (not gated and min_decay >= SCAN_FOLD_MIN_DECAY) else 0), c_int(1 if act else 0), c_int(_dt(proj)),
         o._stream()), "recurrent_scan")
     return out
 
@@ -291,26 +294,80 @@ def head_finish(o_heads, eps: float, out_dtype, *, vdim: int | None = None, stab
 
 
 def qk_norm_write(proj, heads: int, kv_heads: int, dim: int, vdim: int, positions, slots, pool, cache_off: int,
-                  eps: float, temp_coef: float = 0.0, temp_every: float = 1.0, own: bool = True):
+                  eps: float, temp_coef: float = 0.0, temp_every: float = 1.0, own: bool = True, *,
+                  v_heads: int | None = None, q_weight=None, k_weight=None, cos_sin=None, rot_dims: int = 0,
+                  layout: int = 0):
     """Rows of a fused projection, q | k | v (``own``) or q alone (a layer that reads another layer's cache
-    entries): every q and k head is divided by its root mean square (eps inside the root, no weight); q at
-    position p is then multiplied by 1 + temp_coef ln(floor((p + 1) / temp_every) + 1).  k and v go to the paged
-    cache at ``slots`` (< 0: not cached) in the layout ``window_attention`` reads; returns q [T, heads, dim]."""
+    entries): every q and k head is divided by its root mean square (eps inside the root), multiplied by
+    ``q_weight`` / ``k_weight`` (fp32 [dim], shared by the heads) where given, and turned by the rotary table
+    ``cos_sin`` over its first ``rot_dims`` channels (``layout`` 0: pairs (i, i + rot_dims / 2), 1: pairs
+    (2 i, 2 i + 1)); q at position p is then multiplied by 1 + temp_coef ln(floor((p + 1) / temp_every) + 1).
+    k and v go to the paged cache at ``slots`` (< 0: not cached) in the layout ``window_attention`` reads;
+    ``v_heads``: value heads, when fewer than the ``kv_heads`` key heads (several key maps per value head).
+    Returns q [T, heads, dim]."""
+    v_heads = kv_heads if v_heads is None else v_heads
     if not proj.is_cuda:
         return reference.qk_norm_write(proj, heads, kv_heads, dim, vdim, positions, slots, pool, cache_off, eps,
-                                       temp_coef, temp_every, own)
+                                       temp_coef, temp_every, own, v_heads, q_weight, k_weight, cos_sin, rot_dims, layout)
     o = _ops()
     _i32(positions)
+    _f32(q_weight, k_weight, cos_sin)
     t = proj.shape[0]
-    chans = heads * dim + (kv_heads * (dim + vdim) if own else 0)
+    chans = heads * dim + (kv_heads * dim + v_heads * vdim if own else 0)
     assert _rows(proj) and proj.shape[1] >= chans and slots.dtype == torch.int64
-    assert pool.dim() == 2 and pool.stride(1) == 1 and cache_off + window_cache_elems(kv_heads, dim, vdim) <= pool.shape[1]
+    assert pool.dim() == 2 and pool.stride(1) == 1
+    assert cache_off + window_cache_elems(kv_heads, dim, vdim, v_heads) <= pool.shape[1]
+    assert rot_dims == 0 or (cos_sin is not None and cos_sin.shape[1] == rot_dims and rot_dims <= dim)
+    assert all(w is None or w.numel() == dim for w in (q_weight, k_weight))
     q = torch.empty((t, heads, dim), dtype=proj.dtype, device=proj.device)
     o._check(o._kernels().vpsa_qk_norm_write(
         o._p(proj), c_long(proj.stride(0)), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim), c_int(1 if own else 0),
         o._p(positions), o._p(slots), c_float(eps), c_float(temp_coef), c_float(temp_every), o._p(q), _at(pool, cache_off),
-        c_long(pool.stride(0)), c_int(t), c_int(_dt(proj, pool)), o._stream()), "qk_norm_write")
+        c_long(pool.stride(0)), c_int(t), c_int(v_heads), o._p(q_weight), o._p(k_weight), o._p(cos_sin), c_int(rot_dims),
+        c_int(layout), c_int(_dt(proj, pool)), o._stream()), "qk_norm_write")
     return q
+
+
+def pool_blocks(pool, cache_off: int, pool_off: int, kv_heads: int, dim: int, vdim: int, block_tables, row_seq,
+                positions, slots, block: int):
+    """Pooled entries of a windowed attention that sees one mean key and value per block of ``block`` tokens
+    before its window.  For every row of the step that completes a block (position p with (p + 1) % block == 0,
+    cached), the block's keys and values are read back from the pages, averaged in fp32 in position order, and
+    stored as entry b % PAGE of the pooled region (``pool_off`` elements behind the layer's token region, same
+    layout) of the sequence's page b / PAGE, b = p // block.  Call it after the step's keys and values are written
+    and before its attention."""
+    if positions.numel() == 0:
+        return
+    if not pool.is_cuda:
+        return reference.pool_blocks(pool, cache_off, pool_off, kv_heads, dim, vdim, block_tables, row_seq, positions,
+                                     slots, block)
+    o = _ops()
+    _i32(positions, row_seq)
+    assert block_tables.dtype == torch.int32 and block_tables.stride(1) == 1 and slots.dtype == torch.int64
+    assert block >= 1 and pool_off >= window_cache_elems(kv_heads, dim, vdim)
+    assert cache_off + pool_off + window_cache_elems(kv_heads, dim, vdim) <= pool.shape[1]
+    o._check(o._kernels().vpsa_pool_blocks(
+        _at(pool, cache_off), c_long(pool.stride(0)), c_long(pool_off), o._p(block_tables), c_int(block_tables.stride(0)),
+        o._p(row_seq), o._p(positions), o._p(slots), c_int(positions.numel()), c_int(kv_heads * dim),
+        c_int(kv_heads * vdim), c_int(block), c_int(_dt(pool)), o._stream()), "pool_blocks")
+
+
+def diff_heads(u, kv_heads: int, lam: float, eps: float, post: float, out_dtype):
+    """Differential attention's combination.  u fp32 [T, 2 heads, vdim] holds, per key/value group, the first
+    map's outputs of the group's query heads and then the second map's.  Per head o = a1 - lam * a2, divided by its
+    root mean square (eps inside the root), times ``post``; returns [T, heads * vdim] in ``out_dtype``, heads in
+    their natural order."""
+    if not u.is_cuda:
+        return reference.diff_heads(u, kv_heads, lam, eps, post, out_dtype)
+    o = _ops()
+    _f32(u)
+    t, h2, vdim = u.shape
+    assert h2 % 2 == 0 and (h2 // 2) % kv_heads == 0
+    y = torch.empty((t, h2 // 2 * vdim), dtype=out_dtype, device=u.device)
+    o._check(o._kernels().vpsa_diff_heads(o._p(u), o._p(y), c_int(t), c_int(h2 // 2), c_int(kv_heads), c_int(vdim),
+                                          c_float(lam), c_float(eps), c_float(post), c_int(_DT[out_dtype]), o._stream()),
+             "diff_heads")
+    return y
 
 
 def head_rms_norm(o_heads, eps: float, out_dtype, weight=None, gate=None):
@@ -331,9 +388,9 @@ def head_rms_norm(o_heads, eps: float, out_dtype, weight=None, gate=None):
     return y
 
 
-def window_cache_elems(kv_heads: int, dim: int, vdim: int) -> int:
-    """Elements a windowed-attention layer keeps per page."""
-    return PAGE * kv_heads * (dim + vdim)
+def window_cache_elems(kv_heads: int, dim: int, vdim: int, v_heads: int | None = None) -> int:
+    """Elements a windowed-attention layer keeps per page (one region: the tokens', or the pooled blocks')."""
+    return PAGE * (kv_heads * dim + (kv_heads if v_heads is None else v_heads) * vdim)
 
 
 def short_conv_qkv(proj, conv_w, heads: int, kv_heads: int, dim: int, vdim: int, state, state_off: int, row_seq, seq_cu,
@@ -407,10 +464,16 @@ def window_decode_splits(rows: int, kv_heads: int, window: int, keep_first: int,
 
 def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_tables, row_seq, positions, window: int,
                      keep_first: int, scale: float, softcap: float, sink, out=None, tiles=None, splits: int = 1,
-                     own_values: bool = False):
+                     own_values: bool = False, *, chunked: bool = False, pool_block: int = 0, pool_off: int = 0,
+                     maps: int = 1):
     """Query rows q [T, heads, dim] over their sequences' cached keys: row i at position p sees key j when
     j <= p and (p - j < window or j < keep_first).  score = cap * tanh(q . k * scale / cap) (cap 0: none);
-    softmax with ``sink`` [heads] (fp32) in the denominator.  Returns u fp32 [T, heads, kv_heads, vdim]:
+    softmax with ``sink`` [heads] (fp32, or None) in the denominator.  ``chunked``: ``window`` is a chunk size
+    instead, and a row sees the keys of its own chunk (counted from position 0) up to itself.  ``pool_block`` P > 0:
+    beside its window the row also sees the pooled entries (``pool_blocks``, ``pool_off`` elements behind the token
+    region) of every block of P tokens that lies wholly before the window, in the same softmax.  ``maps`` > 1 (with
+    ``own_values``): ``kv_heads`` counts key heads, of which ``maps`` neighbours share one value head.
+    Returns u fp32 [T, heads, kv_heads, vdim]:
     each head's weights applied to the values of every KV head (``mix_heads`` picks and mixes).  With
     ``own_values`` only those of the head's own KV head: u fp32 [T, heads, 1, vdim], the attention output of designs
     without head mixing (a window of at least the context length makes it plain causal attention).
@@ -424,14 +487,20 @@ def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_ta
         out = torch.empty((t, heads, vsets, vdim), dtype=torch.float32, device=q.device)
     if t == 0:
         return out
+    assert maps == 1 or (own_values and kv_heads % maps == 0)
+    assert not pool_block or (keep_first == 0 and not chunked)
     if not q.is_cuda:
         return reference.window_attention(q, pool, cache_off, kv_heads, vdim, block_tables, row_seq, positions, window,
-                                          keep_first, scale, softcap, sink, out, own_values)
+                                          keep_first, scale, softcap, sink, out, own_values, 1 if chunked else 0,
+                                          pool_block, pool_off, maps)
     o = _ops()
     _f32(sink, out)
     _i32(row_seq, positions)
     assert q.is_contiguous() and block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
-    assert heads % kv_heads == 0 and cache_off + window_cache_elems(kv_heads, dim, vdim) <= pool.shape[1]
+    region = window_cache_elems(kv_heads, dim, vdim, kv_heads // maps)
+    assert heads % kv_heads == 0 and cache_off + (pool_off if pool_block else 0) + region <= pool.shape[1]
+    assert not pool_block or (pool_off >= region and (pool_off * pool.element_size()) % 16 == 0)
+    extra = (c_int(1 if chunked else 0), c_int(pool_block), c_long(pool_off), c_int(maps))
     esz = pool.element_size()
     assert (cache_off * esz) % 16 == 0 and (pool.stride(0) * esz) % 16 == 0 and pool.data_ptr() % 16 == 0
     dt = _dt(q, pool)
@@ -452,13 +521,13 @@ def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_ta
             c_int(block_tables.stride(0)), o._p(tiles), o._p(positions), o._p(sink), o._p(out),
             c_int(tiles.shape[0] if tiles is not None else t), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim),
             c_int(window), c_int(keep_first), c_float(scale), c_float(softcap), c_int(splits), o._p(ws_o), o._p(ws_ml),
-            own, o._stream()), "window_attention_mfma")
+            own, *extra, o._stream()), "window_attention_mfma")
         return out
     o._check(o._kernels().vpsa_window_attention(
         o._p(q), c_long(q.stride(0)), _at(pool, cache_off), c_long(pool.stride(0)), o._p(block_tables),
         c_int(block_tables.stride(0)), o._p(row_seq), o._p(positions), o._p(sink), o._p(out), c_int(t), c_int(heads),
         c_int(kv_heads), c_int(dim), c_int(vdim), c_int(window), c_int(keep_first), c_float(scale), c_float(softcap),
-        own, c_int(dt), o._stream()), "window_attention")
+        own, *extra, c_int(dt), o._stream()), "window_attention")
     return out
 
 
