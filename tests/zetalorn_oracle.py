@@ -346,3 +346,23 @@ def save_checkpoint(path, cfg, weights):
         json.dump(cfg, f)
     save_file({k: v.contiguous() for k, v in weights.items()}, os.path.join(path, "model.safetensors"))
     return path
+
+
+# ------------------------------------------------------------------ helpers of the tests
+def forward(cfg, weights, tokens):
+    return run(cfg, weights, tokens)[0]
+
+
+def greedy(cfg, weights, prompt, n_new):
+    toks = list(prompt)
+    for _ in range(n_new):
+        toks.append(int(forward(cfg, weights, toks)[-1].argmax()))
+    return toks[len(prompt):]
+
+
+def row_errors(got, want):
+    """Per row: root mean square of the difference (its mean taken off) over that of the wanted row."""
+    d = got.double() - want.double()
+    d = d - d.mean(-1, keepdim=True)
+    w = want.double() - want.double().mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / w.pow(2).mean(-1).sqrt().clamp_min(1e-30)

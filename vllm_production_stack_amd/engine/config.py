@@ -860,6 +860,49 @@ PRESETS["tiny-pelatar"] = pelatar_config(
 PRESETS["pelatar-bench"] = pelatar_config("pelatar-bench", 32000, 2048, pelatar_stack(2048, 16, 5632, 28, 1024, 4, 4),
                                           max_position_embeddings=32768)
 
+
+def _zx_moe(ff, experts, top, groups, keep, limit=7.0):
+    return {"kind": "moe", "expert": {"ff": ff, "limit": limit},
+            "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}}}
+
+
+def _zx_attention(heads, kv_heads, dim, vdim, chunk, mlp=None):
+    return {"type": "attention", "mlp": mlp,
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "diff": 0.2, "scale": dim ** -0.5,
+                      "mask": {"size": chunk}, "rot": {"base": 10000.0, "dims": dim // 2, "scaling": {"factor": 4.0}}}}
+
+
+def _zx_parallel(heads, kv_heads, dim, vdim, window, pool, r_heads, r_dim, r_vdim, mlp=None):
+    decay = [1.0 - 2.0 ** (-5.0 - 3.0 * i / max(r_heads - 1, 1)) for i in range(r_heads)]
+    return {"type": "parallel", "mlp": mlp,
+            "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
+                               "mask": {"size": window, "pool": pool}, "rot": {"base": 50000.0, "dims": dim}},
+                      "right": {"heads": r_heads, "dim": r_dim, "vdim": r_vdim, "decay": decay}}}
+
+
+def zetalorn_stack(width, heads, experts, unit_ff, top, blocks=1):
+    """Layer list of a Zetalorn at random weights: per block a differential attention layer over chunks of 2048
+    positions and a parallel layer (a window of 1024 positions with blocks of 16 tokens pooled before it, beside a
+    lightning recurrence with half as many heads), both with a routed feed-forward."""
+    routed = _zx_moe(unit_ff, experts, top, 4, 2)
+    out = []
+    for _ in range(blocks):
+        out += [_zx_attention(heads, heads // 4, 128, 128, 2048, routed),
+                _zx_parallel(heads, heads // 4, 128, 128, 1024, 16, heads // 2, 128, 256, routed)]
+    return out
+
+
+# Zetalorn at random weights: a small one for smoke runs, and one with layer shapes of a 2048-wide model whose
+# two layers run twice
+PRESETS["tiny-zetalorn"] = zetalorn_config(
+    "tiny-zetalorn", 512, 128,
+    [_zx_parallel(4, 2, 64, 128, 96, 8, 2, 32, 64, _zx_moe(64, 6, 2, 2, 1)),
+     _zx_attention(4, 2, 64, 128, 160, _zx_moe(64, 4, 2, 1, 1)),
+     _zx_parallel(2, 1, 64, 128, 64, 16, 2, 64, 32)], loop={"start": 0, "stop": 2, "times": 2}, logit_scale=0.5,
+    max_position_embeddings=4096)
+PRESETS["zetalorn-bench"] = zetalorn_config("zetalorn-bench", 32000, 2048, zetalorn_stack(2048, 16, 16, 1024, 4),
+                                            loop={"start": 0, "stop": 2, "times": 2}, logit_scale=0.5)
+
 _ALIASES = {
     "meta-llama/meta-llama-3-8b": "llama-3-8b",
     "meta-llama/meta-llama-3-8b-instruct": "llama-3-8b",
