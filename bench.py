@@ -112,7 +112,7 @@ def parse() -> argparse.Namespace:
                          "VPSA_BENCH_SINGLE_DEVICE=1 (+ --num-gpu-blocks) rehearses either on one card")
     ap.add_argument("--arch-compare", default="",
                     help="instead of the serving benchmark: prefill and decode throughput of this decoder design "
-                         "('zururax', 'revelix', 'pelatar') beside the closest existing design at equal size (benchmarks/arch_compare.py)")
+                         "('zururax', 'revelix', 'pelatar', 'zetalorn') beside the closest existing design at equal size (benchmarks/arch_compare.py)")
     ap.add_argument("--arch-sizes", default="s,m")
     ap.add_argument("--arch-prompt", type=int, default=4096, help="--arch-compare: prompt length")
     ap.add_argument("--arch-prompts", type=int, default=4, help="--arch-compare: prompts per prefill measurement")

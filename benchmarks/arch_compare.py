@@ -1,6 +1,6 @@
 """Prefill and decode throughput of one decoder design beside the closest existing one at equal size.
 
-    python bench.py --arch-compare zururax|revelix|pelatar [--arch-sizes s,m] [--arch-prompt 4096] [--arch-batch 32]
+    python bench.py --arch-compare zururax|revelix|pelatar|zetalorn [--arch-sizes s,m] [--arch-prompt 4096] [--arch-batch 32]
 
 Random weights at layer shapes of real models (a few layers each); both models run through the same
 engine (scheduler, paged pool, HIP-graph decode).  Prefill: prompts of --arch-prompt tokens in chunks of
@@ -32,6 +32,8 @@ def _configs(design: str, size: str):
         return _revelix_configs(size)
     if design == "pelatar":
         return _pelatar_configs(size)
+    if design == "zetalorn":
+        return _zetalorn_configs(size)
     if design != "zururax":
         raise SystemExit(f"--arch-compare: unknown design {design!r}")
 
@@ -102,6 +104,21 @@ def _pelatar_configs(size: str):
                          pelatar_stack(w, z["heads"], ff, z["experts"] - 4, z["ff"], z["top"], 4),
                          max_position_embeddings=32768)
     return new, _revelix_configs(size)[0]
+
+
+def _zetalorn_configs(size: str):
+    """Zetalorn (a differential attention layer over chunks of 2048 positions and a parallel layer: a window of 1024
+    positions with pooled blocks of 16 tokens before it, beside a lightning recurrence; routed clamped units behind
+    both; the pair runs twice, so four layer runs) beside the closest existing design, Pelatar at the same width,
+    depth and head shapes: its attention runs the same tile kernel (one map per head, plain causal), its
+    recurrences the same scan kernel, its routed units the same grouped GEMMs."""
+    from vllm_production_stack_amd.engine.config import zetalorn_config, zetalorn_stack
+
+    z = SIZES[size]
+    new = zetalorn_config(f"zetalorn-{size}", VOCAB, z["width"],
+                          zetalorn_stack(z["width"], z["heads"], z["experts"], z["ff"], z["top"]),
+                          loop={"start": 0, "stop": 2, "times": 2}, logit_scale=0.5, max_position_embeddings=32768)
+    return new, _pelatar_configs(size)[0]
 
 
 def _measure(cfg, a) -> dict:

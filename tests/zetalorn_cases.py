@@ -545,7 +545,8 @@ def check_far_token(device, dtype, cfg, w, tol):
         got = eng.forced_step([(name, toks[200:], [r - 200 for r in rows])], [name]).cpu()
         check_rows(got, want[name], tol, f"prompt {name}")
         other = want["b" if name == "a" else "a"]
-        assert (zo.row_errors(got, want[name]) < zo.row_errors(got, other)).all()  # and it is seen
+        apart = zo.row_errors(want[name], other) > 4 * tol   # (16-bit rounding may be larger than a faint trace)
+        assert (zo.row_errors(got, want[name]) < zo.row_errors(got, other))[apart].all()  # and it is seen
     eng.shutdown()
 
 
