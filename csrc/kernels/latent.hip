@@ -448,47 +448,83 @@ __global__ __launch_bounds__(256) void rmsnorm_add_kernel(float* __restrict__ re
 // with n_i(d) = rmsnorm(d) w_i where a weight w_i is given and d itself otherwise.  Every part is optional: no gate
 // means a plain add, no deltas only the extras (a second stream that re-enters, a vector per pass of a layer loop).
 // d1 in D (the activation dtype, or fp32 for a mixture's sum), d2, gate and y in T.
-template <typename T, typename D>
+template <typename T, typename D, int PER>
 __global__ __launch_bounds__(256) void gated_add_rmsnorm_kernel(
     float* __restrict__ residual, const D* __restrict__ d1, long s1, const float* __restrict__ w1, float c1,
     const T* __restrict__ d2, long s2, const float* __restrict__ w2, float c2, const T* __restrict__ gate, long sg,
     const float* __restrict__ gate_bias, const float* __restrict__ extra, const float* __restrict__ extra_vec,
     const float* __restrict__ w, T* __restrict__ y, int n, float eps) {
+  // PER > 0: rows of up to 256 * PER values; a thread loads every operand of its values once, all loads in flight
+  // together before the first sum (a few rows per launch are bound by that chain's latency, not by bytes).
+  // PER = 0: any width, operands are read again where needed.
   __shared__ float red[4];
+  constexpr int P = PER > 0 ? PER : 1;
   const long row = blockIdx.x;
   float* r = residual + row * n;
+  float a1[P], a2[P], rv[P], gv[P], wv[P];
+  float q1 = 0.f, q2 = 0.f;
+  if (PER > 0) {
+#pragma unroll
+    for (int k = 0; k < P; ++k) {
+      const int i = threadIdx.x + 256 * k;
+      const bool in = i < n;
+      a1[k] = (d1 && in) ? Conv<D>::ld(d1 + row * s1 + i) : 0.f;
+      a2[k] = (d2 && in) ? Conv<T>::ld(d2 + row * s2 + i) : 0.f;
+      gv[k] = (gate && in) ? Conv<T>::ld(gate + row * sg + i) + (gate_bias ? gate_bias[i] : 0.f) : 0.f;
+      rv[k] = in ? r[i] + (extra ? extra[row * n + i] : 0.f) + (extra_vec ? extra_vec[i] : 0.f) : 0.f;
+      wv[k] = (y && in) ? w[i] : 0.f;
+      q1 += a1[k] * a1[k];
+      q2 += a2[k] * a2[k];
+      if (in) {  // the deltas' own weights: applied here, the norms' factors follow below
+        if (d1 && w1) a1[k] *= w1[i];
+        if (d2 && w2) a2[k] *= w2[i];
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < n; i += 256) {
+      const float u = d1 ? Conv<D>::ld(d1 + row * s1 + i) : 0.f, v = d2 ? Conv<T>::ld(d2 + row * s2 + i) : 0.f;
+      q1 += u * u;
+      q2 += v * v;
+    }
+  }
   float f1 = c1, f2 = c2;
-  if (d1 && w1) {
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < n; i += 256) {
-      const float v = Conv<D>::ld(d1 + row * s1 + i);
-      ss += v * v;
-    }
-    f1 = c1 / sqrtf(block_sum(ss, red) / (float)n + eps);
-  }
-  if (d2 && w2) {
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < n; i += 256) {
-      const float v = Conv<T>::ld(d2 + row * s2 + i);
-      ss += v * v;
-    }
-    f2 = c2 / sqrtf(block_sum(ss, red) / (float)n + eps);
-  }
+  if (d1 && w1) f1 = c1 / sqrtf(block_sum(q1, red) / (float)n + eps);
+  if (d2 && w2) f2 = c2 / sqrtf(block_sum(q2, red) / (float)n + eps);
   float ss = 0.f;
-  for (int i = threadIdx.x; i < n; i += 256) {
-    float d = 0.f;
-    if (d1) d += Conv<D>::ld(d1 + row * s1 + i) * f1 * (w1 ? w1[i] : 1.f);
-    if (d2) d += Conv<T>::ld(d2 + row * s2 + i) * f2 * (w2 ? w2[i] : 1.f);
-    if (gate) d *= sigmoidf(Conv<T>::ld(gate + row * sg + i) + (gate_bias ? gate_bias[i] : 0.f));
-    float v = r[i] + d;
-    if (extra) v += extra[row * n + i];
-    if (extra_vec) v += extra_vec[i];
-    r[i] = v;  // read back below by the same thread
-    ss += v * v;
+  if (PER > 0) {
+#pragma unroll
+    for (int k = 0; k < P; ++k) {
+      const int i = threadIdx.x + 256 * k;
+      float d = a1[k] * f1 + a2[k] * f2;
+      if (gate) d *= sigmoidf(gv[k]);
+      rv[k] += d;
+      if (i < n) r[i] = rv[k];
+      ss += rv[k] * rv[k];
+    }
+  } else {
+    for (int i = threadIdx.x; i < n; i += 256) {
+      float d = 0.f;
+      if (d1) d += Conv<D>::ld(d1 + row * s1 + i) * f1 * (w1 ? w1[i] : 1.f);
+      if (d2) d += Conv<T>::ld(d2 + row * s2 + i) * f2 * (w2 ? w2[i] : 1.f);
+      if (gate) d *= sigmoidf(Conv<T>::ld(gate + row * sg + i) + (gate_bias ? gate_bias[i] : 0.f));
+      float x = r[i] + d;
+      if (extra) x += extra[row * n + i];
+      if (extra_vec) x += extra_vec[i];
+      r[i] = x;  // read back below by the same thread
+      ss += x * x;
+    }
   }
   if (!y) return;
   const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
-  for (int i = threadIdx.x; i < n; i += 256) Conv<T>::st(y + row * n + i, r[i] * inv * w[i]);
+  if (PER > 0) {
+#pragma unroll
+    for (int k = 0; k < P; ++k) {
+      const int i = threadIdx.x + 256 * k;
+      if (i < n) Conv<T>::st(y + row * n + i, rv[k] * inv * wv[k]);
+    }
+  } else {
+    for (int i = threadIdx.x; i < n; i += 256) Conv<T>::st(y + row * n + i, r[i] * inv * w[i]);
+  }
 }
 
 // x [rows, 2 inter] = gate | up  ->  act(gate) * up;  kind 0: silu, 1: gelu in its tanh form
@@ -661,13 +697,19 @@ VPSA_EXPORT int vpsa_gated_add_rmsnorm(float* residual, const void* d1, long s1,
   if (rows <= 0) return 0;
   if (dtype != 0 && dtype != 1) return -2;
   if (y && !w) return -1;
-#define GA(T, D)                                                                                                     \
-  gated_add_rmsnorm_kernel<T, D><<<rows, 256, 0, st>>>(residual, (const D*)d1, s1, w1, c1, (const T*)d2, s2, w2, c2, \
-                                                       (const T*)gate, sg, gate_bias, extra, extra_vec, w, (T*)y, n, eps)
-  if (dtype == 1) GA(float, float);
-  else if (d1_f32) GA(bf16_t, float);
-  else GA(bf16_t, bf16_t);
+#define GA_P(T, D, P)                                                                                                   \
+  gated_add_rmsnorm_kernel<T, D, P><<<rows, 256, 0, st>>>(residual, (const D*)d1, s1, w1, c1, (const T*)d2, s2, w2, c2, \
+                                                          (const T*)gate, sg, gate_bias, extra, extra_vec, w, (T*)y, n, eps)
+#define GA(T, D)                         \
+  if (n <= 1024) GA_P(T, D, 4);          \
+  else if (n <= 2048) GA_P(T, D, 8);     \
+  else if (n <= 4096) GA_P(T, D, 16);    \
+  else GA_P(T, D, 0)
+  if (dtype == 1) { GA(float, float); }
+  else if (d1_f32) { GA(bf16_t, float); }
+  else { GA(bf16_t, bf16_t); }
 #undef GA
+#undef GA_P
   return 0;
 }
 

@@ -462,7 +462,7 @@ __global__ __launch_bounds__(256) void mlstm_prepare_kernel(const T* __restrict_
   }
 }
 
-// One workgroup per row, a wave per head in turn.  Row = q [heads * dim] (| k [kv_heads * dim] | v [v_heads * vdim]
+// A workgroup per row and run of four heads (blockIdx.y), a wave per head.  Row = q [heads * dim] (| k [kv_heads * dim] | v [v_heads * vdim]
 // when the layer owns its cache entries).  q and k heads are divided by their root mean square (eps inside the
 // root), multiplied by a weight per channel where one is given (qw / kw, shared by the heads), and turned by the
 // rotary table over their first rot_dims channels (cos_sin null: no rotation); q is then multiplied by
@@ -486,7 +486,8 @@ __global__ __launch_bounds__(256) void qk_norm_write_kernel(const T* __restrict_
   if (coef != 0.f) temp = 1.f + coef * logf((float)floor((double)(p + 1) / (double)every) + 1.f);
   const long slot = own ? slots[row] : -1;
   const int nk = kv_heads * dim;
-  for (int hh = wave; hh < heads + (own ? kv_heads : 0); hh += 4) {
+  const int hh = blockIdx.y * 4 + wave;
+  if (hh < heads + (own ? kv_heads : 0)) {
     const T* src = pr + (long)hh * dim;  // k heads follow the q heads
     float ss = 0.f;
     for (int i = lane; i < dim; i += 64) {
@@ -509,38 +510,57 @@ __global__ __launch_bounds__(256) void qk_norm_write_kernel(const T* __restrict_
   if (slot >= 0) {
     const T* vs = pr + (long)heads * dim + nk;
     T* dst = cache + (slot / PAGE) * page_stride + (long)PAGE * nk + (slot % PAGE);
-    for (int c = threadIdx.x; c < v_heads * vdim; c += 256) dst[(long)c * PAGE] = vs[c];
+    for (int c = blockIdx.y * 256 + threadIdx.x; c < v_heads * vdim; c += gridDim.y * 256) dst[(long)c * PAGE] = vs[c];
   }
 }
 
-// Pooled entries of a windowed attention that also sees a mean key and value per block of `pool` tokens.  One
-// workgroup per row of the step: a row at position p with (p + 1) % pool == 0 completes block b = p / pool; the
+// Pooled entries of a windowed attention that also sees a mean key and value per block of `pool` tokens.  A row
+// of the step at position p with (p + 1) % pool == 0 completes block b = p / pool; the
 // block's keys and values are read back from the pages (as the cache holds them, whichever step wrote them), summed
 // in position order in fp32 and divided by pool, and stored as entry b % PAGE of the pooled region (pool_off
 // elements behind the token region, same layout) of the sequence's page b / PAGE.
+constexpr int POOL_ROWS = 16;  // rows of the step a workgroup looks at
+
 template <typename T>
 __global__ __launch_bounds__(256) void pool_blocks_kernel(T* __restrict__ cache, long page_stride, long pool_off,
                                                           const int* __restrict__ block_tables, int bt_stride,
                                                           const int* __restrict__ row_seq,
                                                           const int* __restrict__ positions,
-                                                          const long* __restrict__ slots, int nk, int nv, int pool) {
-  const long row = blockIdx.x;
-  const int p = positions[row];
-  if (slots[row] < 0 || (p + 1) % pool != 0) return;
-  const int seq = row_seq ? row_seq[row] : (int)row;
-  const int* bt = block_tables + (long)seq * bt_stride;
-  const int b = p / pool, j0 = b * pool;
-  T* dst = cache + (long)bt[b / PAGE] * page_stride + pool_off;
-  const float inv = 1.f / (float)pool;
-  for (int c = threadIdx.x; c < nk + nv; c += 256) {
+                                                          const long* __restrict__ slots, int rows, int nk, int nv,
+                                                          int pool) {
+  // blockIdx.x: a run of POOL_ROWS rows, of which those that complete a block are worked on one after the other
+  // (most workgroups find none or one); blockIdx.y: a run of 256 channels (keys first, then values).  A thread owns
+  // one channel and walks the block's tokens page by page (a page's tokens are a strided run for a key channel, a
+  // contiguous one for a value channel), summing in position order.
+  __shared__ int todo[POOL_ROWS];
+  const int tid = threadIdx.x;
+  if (tid < POOL_ROWS) {
+    const long row = (long)blockIdx.x * POOL_ROWS + tid;
+    int p = -1;
+    if (row < rows && slots[row] >= 0 && (positions[row] + 1) % pool == 0) p = positions[row];
+    todo[tid] = p;
+  }
+  __syncthreads();
+  const int c = blockIdx.y * 256 + tid;
+  if (c >= nk + nv) return;
+  const bool is_k = c < nk;
+  const long off = is_k ? c : (long)PAGE * nk + (long)(c - nk) * PAGE, step = is_k ? nk : 1;
+  for (int k = 0; k < POOL_ROWS; ++k) {
+    const int p = todo[k];
+    if (p < 0) continue;
+    const long row = (long)blockIdx.x * POOL_ROWS + k;
+    const int seq = row_seq ? row_seq[row] : (int)row;
+    const int* bt = block_tables + (long)seq * bt_stride;
+    const int b = p / pool, j0 = b * pool;
     float acc = 0.f;
-    for (int j = j0; j <= p; ++j) {
-      const T* src = cache + (long)bt[j / PAGE] * page_stride;
-      acc += c < nk ? Cv<T>::ld(src + (long)(j % PAGE) * nk + c)
-                    : Cv<T>::ld(src + (long)PAGE * nk + (long)(c - nk) * PAGE + j % PAGE);
+    for (int pg = j0 / PAGE; pg <= p / PAGE; ++pg) {
+      const int a = max(j0, pg * PAGE) % PAGE, e = min(p, pg * PAGE + PAGE - 1) % PAGE;
+      const T* src = cache + (long)bt[pg] * page_stride + off;
+#pragma unroll 8
+      for (int r = a; r <= e; ++r) acc += Cv<T>::ld(src + r * step);
     }
-    if (c < nk) Cv<T>::st(dst + (long)(b % PAGE) * nk + c, acc * inv);
-    else Cv<T>::st(dst + (long)PAGE * nk + (long)(c - nk) * PAGE + b % PAGE, acc * inv);
+    T* dst = cache + (long)bt[b / PAGE] * page_stride + pool_off + off;
+    Cv<T>::st(dst + (b % PAGE) * step, acc / (float)pool);
   }
 }
 
@@ -600,6 +620,41 @@ __global__ __launch_bounds__(256) void head_rms_kernel(const float* __restrict__
     inv = 1.f / sqrtf(ss / (float)vdim + eps);
   }
   for (int c = lane; c < vdim; c += 64) {
+    float v = op[c] * pre * inv;
+    if (w) v *= w[w_heads ? head * vdim + c : c];
+    if (gate) {
+      const float g = Cv<T>::ld(gate + row * g_stride + head * vdim + c);
+      v *= gate_act == 0 ? g * sigm(g) : sigm(g);
+    }
+    Cv<T>::st(y + pair * vdim + c, v);
+  }
+}
+
+// The same with one workgroup per (row, head), for heads of a thousand channels and more (all heads of a mixer
+// normed together, say), where a single wave per head would walk its channels alone.
+template <typename T>
+__global__ __launch_bounds__(256) void head_rms_wide_kernel(const float* __restrict__ o, int ostride,
+                                                            const float* __restrict__ stab, int unit,
+                                                            const float* __restrict__ w, int w_heads,
+                                                            const T* __restrict__ gate, long g_stride, int gate_act,
+                                                            T* __restrict__ y, int heads, int vdim, float eps) {
+  __shared__ float red[4];
+  const long pair = blockIdx.x;
+  const long row = pair / heads;
+  const int head = (int)(pair - row * heads);
+  const float* op = o + pair * ostride;
+  float pre = 1.f;
+  if (stab) pre = 1.f / (fmaxf(fabsf(op[vdim]), expf(-stab[pair])) + 1e-6f);
+  float inv = 1.f;
+  if (unit) {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < vdim; c += 256) {
+      const float v = op[c] * pre;
+      ss += v * v;
+    }
+    inv = 1.f / sqrtf(blk_sum(ss, red) / (float)vdim + eps);
+  }
+  for (int c = threadIdx.x; c < vdim; c += 256) {
     float v = op[c] * pre * inv;
     if (w) v *= w[w_heads ? head * vdim + c : c];
     if (gate) {
@@ -1271,6 +1326,11 @@ VPSA_EXPORT int vpsa_head_finish(const float* o, int ostride, const float* stab,
   const long pairs = (long)rows * heads;
   if (pairs <= 0) return 0;
   if (ostride < vdim + (stab ? 1 : 0)) return 2;
+  if (vdim >= 1024) {
+    SM_DISPATCH(dt, (head_rms_wide_kernel<T><<<(unsigned)pairs, 256, 0, stream>>>(
+                        o, ostride, stab, unit, w, w_heads, (const T*)gate, g_stride, gate_act, (T*)y, heads, vdim, eps)));
+    return 0;
+  }
   SM_DISPATCH(dt, (head_rms_kernel<T><<<(unsigned)((pairs + 3) / 4), 256, 0, stream>>>(
                       o, ostride, stab, unit, w, w_heads, (const T*)gate, g_stride, gate_act, (T*)y, pairs, heads, vdim,
                       eps)));
@@ -1291,7 +1351,8 @@ VPSA_EXPORT int vpsa_qk_norm_write(const void* proj, long p_stride, int heads, i
   if (rows <= 0) return 0;
   if (coef != 0.f && !(every > 0.f)) return 2;
   if (rot_dims < 0 || rot_dims > dim || rot_dims % 2 || (rot_dims && !cos_sin) || v_heads < 1) return 3;
-  SM_DISPATCH(dt, (qk_norm_write_kernel<T><<<rows, 256, 0, stream>>>(
+  const int head_runs = (heads + (own ? kv_heads : 0) + 3) / 4;
+  SM_DISPATCH(dt, (qk_norm_write_kernel<T><<<dim3(rows, head_runs), 256, 0, stream>>>(
                       (const T*)proj, p_stride, heads, kv_heads, dim, vdim, own, positions, slots, eps, coef, every,
                       (T*)q_out, (T*)cache, page_stride, v_heads, qw, kw, rot_dims ? cos_sin : nullptr, rot_dims, layout)));
   return 0;
@@ -1303,8 +1364,9 @@ VPSA_EXPORT int vpsa_pool_blocks(void* cache, long page_stride, long pool_off, c
                                  int pool, int dt, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (pool < 1 || pool_off < (long)PAGE * (nk + nv)) return 2;
-  SM_DISPATCH(dt, (pool_blocks_kernel<T><<<rows, 256, 0, stream>>>((T*)cache, page_stride, pool_off, block_tables, bt_stride,
-                                                                   row_seq, positions, slots, nk, nv, pool)));
+  SM_DISPATCH(dt, (pool_blocks_kernel<T><<<dim3((rows + POOL_ROWS - 1) / POOL_ROWS, (nk + nv + 255) / 256), 256, 0, stream>>>(
+                      (T*)cache, page_stride, pool_off, block_tables, bt_stride, row_seq, positions, slots, rows, nk, nv,
+                      pool)));
   return 0;
 }
 
