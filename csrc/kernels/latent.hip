@@ -448,81 +448,141 @@ __global__ __launch_bounds__(256) void rmsnorm_add_kernel(float* __restrict__ re
 // with n_i(d) = rmsnorm(d) w_i where a weight w_i is given and d itself otherwise.  Every part is optional: no gate
 // means a plain add, no deltas only the extras (a second stream that re-enters, a vector per pass of a layer loop).
 // d1 in D (the activation dtype, or fp32 for a mixture's sum), d2, gate and y in T.
-template <typename T, typename D, int PER>
+__device__ __forceinline__ void ld8(const float* p, float* v) {
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = a[e], v[4 + e] = b[e];
+}
+__device__ __forceinline__ void ld8(const bf16_t* p, float* v) {
+  const u32x4 a = *reinterpret_cast<const u32x4*>(p);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[2 * e] = bf16lo(a[e]), v[2 * e + 1] = bf16hi(a[e]);
+}
+__device__ __forceinline__ void st8(float* p, const float* v) {
+  *reinterpret_cast<f32x4*>(p) = (f32x4){v[0], v[1], v[2], v[3]};
+  *reinterpret_cast<f32x4*>(p + 4) = (f32x4){v[4], v[5], v[6], v[7]};
+}
+__device__ __forceinline__ void st8(bf16_t* p, const float* v) {
+  *reinterpret_cast<u32x4*>(p) = (u32x4){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]),
+                                         pack_bf16x2(v[6], v[7])};
+}
+
+// K > 0: rows of up to 2048 K values, a multiple of 8, every operand on 16-byte boundaries: a thread owns runs of 8
+// neighbouring values, loads every operand once with 16-byte loads and keeps the new stream in registers.
+// K = 0: any width and alignment, value by value, operands read again where needed.
+template <typename T, typename D, int K>
 __global__ __launch_bounds__(256) void gated_add_rmsnorm_kernel(
     float* __restrict__ residual, const D* __restrict__ d1, long s1, const float* __restrict__ w1, float c1,
     const T* __restrict__ d2, long s2, const float* __restrict__ w2, float c2, const T* __restrict__ gate, long sg,
     const float* __restrict__ gate_bias, const float* __restrict__ extra, const float* __restrict__ extra_vec,
     const float* __restrict__ w, T* __restrict__ y, int n, float eps) {
-  // PER > 0: rows of up to 256 * PER values; a thread loads every operand of its values once, all loads in flight
-  // together before the first sum (a few rows per launch are bound by that chain's latency, not by bytes).
-  // PER = 0: any width, operands are read again where needed.
   __shared__ float red[4];
-  constexpr int P = PER > 0 ? PER : 1;
   const long row = blockIdx.x;
   float* r = residual + row * n;
-  float a1[P], a2[P], rv[P], gv[P], wv[P];
-  float q1 = 0.f, q2 = 0.f;
-  if (PER > 0) {
+  if constexpr (K > 0) {
+    float a1[K][8], a2[K][8], x[K][8];
+    float q1 = 0.f, q2 = 0.f;
 #pragma unroll
-    for (int k = 0; k < P; ++k) {
-      const int i = threadIdx.x + 256 * k;
-      const bool in = i < n;
-      a1[k] = (d1 && in) ? Conv<D>::ld(d1 + row * s1 + i) : 0.f;
-      a2[k] = (d2 && in) ? Conv<T>::ld(d2 + row * s2 + i) : 0.f;
-      gv[k] = (gate && in) ? Conv<T>::ld(gate + row * sg + i) + (gate_bias ? gate_bias[i] : 0.f) : 0.f;
-      rv[k] = in ? r[i] + (extra ? extra[row * n + i] : 0.f) + (extra_vec ? extra_vec[i] : 0.f) : 0.f;
-      wv[k] = (y && in) ? w[i] : 0.f;
-      q1 += a1[k] * a1[k];
-      q2 += a2[k] * a2[k];
-      if (in) {  // the deltas' own weights: applied here, the norms' factors follow below
-        if (d1 && w1) a1[k] *= w1[i];
-        if (d2 && w2) a2[k] *= w2[i];
+    for (int k = 0; k < K; ++k) {
+      const int i = (threadIdx.x + 256 * k) * 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) a1[k][e] = a2[k][e] = 0.f;
+      if (i < n) {
+        if (d1) ld8(d1 + row * s1 + i, a1[k]);
+        if (d2) ld8(d2 + row * s2 + i, a2[k]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q1 += a1[k][e] * a1[k][e], q2 += a2[k][e] * a2[k][e];
+    }
+    float f1 = c1, f2 = c2;
+    if (d1 && w1) f1 = c1 / sqrtf(block_sum(q1, red) / (float)n + eps);
+    if (d2 && w2) f2 = c2 / sqrtf(block_sum(q2, red) / (float)n + eps);
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int i = (threadIdx.x + 256 * k) * 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[k][e] = 0.f;
+      if (i < n) {
+        float t[8], u[8];
+        ld8(r + i, x[k]);
+        if (d1 && w1) {
+          ld8(w1 + i, t);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) a1[k][e] *= t[e];
+        }
+        if (d2 && w2) {
+          ld8(w2 + i, t);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) a2[k][e] *= t[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] = a1[k][e] * f1 + a2[k][e] * f2;
+        if (gate) {
+          ld8(gate + row * sg + i, u);
+          if (gate_bias) {
+            float b[8];
+            ld8(gate_bias + i, b);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) u[e] += b[e];
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) t[e] *= sigmoidf(u[e]);
+        }
+        if (extra) {
+          ld8(extra + row * n + i, u);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) t[e] += u[e];
+        }
+        if (extra_vec) {
+          ld8(extra_vec + i, u);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) t[e] += u[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[k][e] += t[e];
+        if (d1 || d2 || extra || extra_vec) st8(r + i, x[k]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += x[k][e] * x[k][e];
+    }
+    if (!y) return;
+    const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int i = (threadIdx.x + 256 * k) * 8;
+      if (i < n) {
+        float t[8];
+        ld8(w + i, t);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] *= x[k][e] * inv;
+        st8(y + row * n + i, t);
       }
     }
   } else {
+    float q1 = 0.f, q2 = 0.f;
     for (int i = threadIdx.x; i < n; i += 256) {
       const float u = d1 ? Conv<D>::ld(d1 + row * s1 + i) : 0.f, v = d2 ? Conv<T>::ld(d2 + row * s2 + i) : 0.f;
       q1 += u * u;
       q2 += v * v;
     }
-  }
-  float f1 = c1, f2 = c2;
-  if (d1 && w1) f1 = c1 / sqrtf(block_sum(q1, red) / (float)n + eps);
-  if (d2 && w2) f2 = c2 / sqrtf(block_sum(q2, red) / (float)n + eps);
-  float ss = 0.f;
-  if (PER > 0) {
-#pragma unroll
-    for (int k = 0; k < P; ++k) {
-      const int i = threadIdx.x + 256 * k;
-      float d = a1[k] * f1 + a2[k] * f2;
-      if (gate) d *= sigmoidf(gv[k]);
-      rv[k] += d;
-      if (i < n) r[i] = rv[k];
-      ss += rv[k] * rv[k];
-    }
-  } else {
+    float f1 = c1, f2 = c2;
+    if (d1 && w1) f1 = c1 / sqrtf(block_sum(q1, red) / (float)n + eps);
+    if (d2 && w2) f2 = c2 / sqrtf(block_sum(q2, red) / (float)n + eps);
+    float ss = 0.f;
     for (int i = threadIdx.x; i < n; i += 256) {
       float d = 0.f;
       if (d1) d += Conv<D>::ld(d1 + row * s1 + i) * f1 * (w1 ? w1[i] : 1.f);
       if (d2) d += Conv<T>::ld(d2 + row * s2 + i) * f2 * (w2 ? w2[i] : 1.f);
       if (gate) d *= sigmoidf(Conv<T>::ld(gate + row * sg + i) + (gate_bias ? gate_bias[i] : 0.f));
-      float x = r[i] + d;
-      if (extra) x += extra[row * n + i];
-      if (extra_vec) x += extra_vec[i];
-      r[i] = x;  // read back below by the same thread
-      ss += x * x;
+      float v = r[i] + d;
+      if (extra) v += extra[row * n + i];
+      if (extra_vec) v += extra_vec[i];
+      r[i] = v;  // read back below by the same thread
+      ss += v * v;
     }
-  }
-  if (!y) return;
-  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
-  if (PER > 0) {
-#pragma unroll
-    for (int k = 0; k < P; ++k) {
-      const int i = threadIdx.x + 256 * k;
-      if (i < n) Conv<T>::st(y + row * n + i, rv[k] * inv * wv[k]);
-    }
-  } else {
+    if (!y) return;
+    const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
     for (int i = threadIdx.x; i < n; i += 256) Conv<T>::st(y + row * n + i, r[i] * inv * w[i]);
   }
 }
@@ -700,10 +760,14 @@ VPSA_EXPORT int vpsa_gated_add_rmsnorm(float* residual, const void* d1, long s1,
 #define GA_P(T, D, P)                                                                                                   \
   gated_add_rmsnorm_kernel<T, D, P><<<rows, 256, 0, st>>>(residual, (const D*)d1, s1, w1, c1, (const T*)d2, s2, w2, c2, \
                                                           (const T*)gate, sg, gate_bias, extra, extra_vec, w, (T*)y, n, eps)
-#define GA(T, D)                         \
-  if (n <= 1024) GA_P(T, D, 4);          \
-  else if (n <= 2048) GA_P(T, D, 8);     \
-  else if (n <= 4096) GA_P(T, D, 16);    \
+  // 16-byte loads need every operand's rows on 16-byte boundaries
+  auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  const bool vec = n % 8 == 0 && s1 % 8 == 0 && s2 % 8 == 0 && sg % 8 == 0 && al(residual) && al(d1) && al(w1) && al(d2) &&
+                   al(w2) && al(gate) && al(gate_bias) && al(extra) && al(extra_vec) && al(w) && al(y);
+#define GA(T, D)                                 \
+  if (vec && n <= 2048) GA_P(T, D, 1);           \
+  else if (vec && n <= 4096) GA_P(T, D, 2);      \
+  else if (vec && n <= 8192) GA_P(T, D, 4);      \
   else GA_P(T, D, 0)
   if (dtype == 1) { GA(float, float); }
   else if (d1_f32) { GA(bf16_t, float); }

@@ -462,7 +462,7 @@ __global__ __launch_bounds__(256) void mlstm_prepare_kernel(const T* __restrict_
   }
 }
 
-// A workgroup per row and run of four heads (blockIdx.y), a wave per head.  Row = q [heads * dim] (| k [kv_heads * dim] | v [v_heads * vdim]
+// A workgroup per row, a wave per head in turn.  Row = q [heads * dim] (| k [kv_heads * dim] | v [v_heads * vdim]
 // when the layer owns its cache entries).  q and k heads are divided by their root mean square (eps inside the
 // root), multiplied by a weight per channel where one is given (qw / kw, shared by the heads), and turned by the
 // rotary table over their first rot_dims channels (cos_sin null: no rotation); q is then multiplied by
@@ -486,8 +486,8 @@ __global__ __launch_bounds__(256) void qk_norm_write_kernel(const T* __restrict_
   if (coef != 0.f) temp = 1.f + coef * logf((float)floor((double)(p + 1) / (double)every) + 1.f);
   const long slot = own ? slots[row] : -1;
   const int nk = kv_heads * dim;
-  const int hh = blockIdx.y * 4 + wave;
-  if (hh < heads + (own ? kv_heads : 0)) {
+  // (a few rows per launch: the heads are spread over blockIdx.y; many rows: one workgroup walks them in turn)
+  for (int hh = blockIdx.y * 4 + wave; hh < heads + (own ? kv_heads : 0); hh += gridDim.y * 4) {
     const T* src = pr + (long)hh * dim;  // k heads follow the q heads
     float ss = 0.f;
     for (int i = lane; i < dim; i += 64) {
@@ -1351,7 +1351,7 @@ VPSA_EXPORT int vpsa_qk_norm_write(const void* proj, long p_stride, int heads, i
   if (rows <= 0) return 0;
   if (coef != 0.f && !(every > 0.f)) return 2;
   if (rot_dims < 0 || rot_dims > dim || rot_dims % 2 || (rot_dims && !cos_sin) || v_heads < 1) return 3;
-  const int head_runs = (heads + (own ? kv_heads : 0) + 3) / 4;
+  const int head_runs = rows <= 512 ? (heads + (own ? kv_heads : 0) + 3) / 4 : 1;
   SM_DISPATCH(dt, (qk_norm_write_kernel<T><<<dim3(rows, head_runs), 256, 0, stream>>>(
                       (const T*)proj, p_stride, heads, kv_heads, dim, vdim, own, positions, slots, eps, coef, every,
                       (T*)q_out, (T*)cache, page_stride, v_heads, qw, kw, rot_dims ? cos_sin : nullptr, rot_dims, layout)));

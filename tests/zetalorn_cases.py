@@ -102,16 +102,17 @@ def case_gated_residual(dev, dtype, tol):
     dt = DTYPES[dtype]
     g = torch.Generator().manual_seed(0)
     eps = 1e-5
-    for n in (5, 48, 300):
+    for n in (5, 48, 300, 2304, 4104):   # widths that take 16-byte loads (in one, two and four runs per thread) and not
+        at = 8 if n % 8 == 0 else 3
         res = torch.randn(7, n, generator=g) * 2
         w = torch.rand(n, generator=g) + 0.5
         d1 = (torch.randn(7, n, generator=g) * 3).to(dt)
         d2 = (torch.randn(7, n, generator=g) * 0.1).to(dt)
         w1, w2 = torch.rand(n, generator=g) + 0.5, torch.rand(n, generator=g) + 0.5
-        wide = (torch.randn(7, 2 * n + 3, generator=g) * 2).to(dt)   # the gate is a view of a wider projection
+        wide = (torch.randn(7, 2 * n + 8, generator=g) * 2).to(dt)   # the gate is a view of a wider projection
         bias = torch.randn(n, generator=g)
         extra, vec = torch.randn(7, n, generator=g), torch.randn(n, generator=g)
-        sg = zo.sigmoid(wide[:, 3:3 + n].double() + bias.double())
+        sg = zo.sigmoid(wide[:, at:at + n].double() + bias.double())
         cases = {
             "one gated delta": ([(d1, None, 1.0)], True, None, None, sg * d1.double()),
             "a delta in 32 bits": ([(d1.float() * 1e-3, None, 1.0)], True, None, None, sg * d1.float().double() * 1e-3),
@@ -126,14 +127,14 @@ def case_gated_residual(dev, dtype, tol):
         for name, (deltas, gated, ex, ve, add) in cases.items():
             r = res.clone().to(dev)
             deltas = [(d.to(dev), None if nw is None else nw.to(dev), c) for d, nw, c in deltas]
-            y = ops.gated_add_rms_norm(r, deltas, wide.to(dev)[:, 3:3 + n] if gated else None, bias.to(dev) if gated else None,
+            y = ops.gated_add_rms_norm(r, deltas, wide.to(dev)[:, at:at + n] if gated else None, bias.to(dev) if gated else None,
                                        w.to(dev), eps, dt, extra=None if ex is None else ex.to(dev),
                                        extra_vec=None if ve is None else ve.to(dev))
             want = res.double() + add
             close(r, want, 2e-6, f"{name}: stream, width {n}")
             close(y, zo.rms(want, eps) * w.double(), tol, f"{name}: normed, width {n}")
             r2 = res.clone().to(dev)
-            assert ops.gated_add_rms_norm(r2, deltas, wide.to(dev)[:, 3:3 + n] if gated else None,
+            assert ops.gated_add_rms_norm(r2, deltas, wide.to(dev)[:, at:at + n] if gated else None,
                                           bias.to(dev) if gated else None, None, eps, dt,
                                           extra=None if ex is None else ex.to(dev),
                                           extra_vec=None if ve is None else ve.to(dev), want_out=False) is None
