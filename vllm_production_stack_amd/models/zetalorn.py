@@ -328,12 +328,12 @@ class ZetalornModel:
         """The mixture's output for rows h, fp32."""
         f: FeedForwardSpec = lw.spec.mlp
         t = h.shape[0]
-        logits = F.linear(h.float(), lw.router)  # a true fp32 product
-        w, ids, _ = ops.group_topk(logits, f.experts, f.groups, f.keep, f.top, 1.0, normalize=f.norm_topk)
-        out = torch.zeros((t, h.shape[1]), dtype=torch.float32, device=h.device)
+        # the logits are a true fp32 product of the rows as they are
+        w, ids, _ = ops.route_group_topk(h, lw.router, f.experts, f.groups, f.keep, f.top, 1.0, normalize=f.norm_topk)
+        out = torch.empty((t, h.shape[1]), dtype=torch.float32, device=h.device)
         if ops.moe_glu_grouped_supported(h, lw.w13, lw.w2):
             ys, pos = ops.moe_glu_grouped(h, lw.w13, lw.w2, ids, f.limit, GLU_ALPHA, GLU_UP_BIAS)
-            return ops.moe_finish(out, ys, w, pos)
+            return ops.moe_finish(out, ys, w, pos, overwrite=True)
         # the CPU, fp32, and shapes the grouped kernel does not tile: unit by unit on the sorted rows
         offsets, pos, sorted_tok = ops.moe_align(ids, f.experts)
         xs = ops.gather_rows(h, sorted_tok)
@@ -344,7 +344,7 @@ class ZetalornModel:
             if b > a:
                 act = ops.glu_clamp(F.linear(xs[a:b], lw.w13[e]), f.limit, GLU_ALPHA, GLU_UP_BIAS)
                 torch.matmul(act, lw.w2[e].t(), out=ys[a:b])
-        return ops.moe_finish(out, ys, w, pos)
+        return ops.moe_finish(out, ys, w, pos, overwrite=True)
 
     # ------------------------------------------------------------------ forward
     def _norm(self, x, pending: Pending | None, weight, **extras):
