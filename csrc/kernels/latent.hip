@@ -284,16 +284,11 @@ __global__ __launch_bounds__(256) void glu_clamp_kernel(const T* __restrict__ x,
 // form `groups` equal runs of neighbours; a group scores the sum of its two largest scores (its
 // only one for groups of one); experts outside the `keep` best groups cannot be chosen.  Weights
 // are the chosen scores times route_scale (not renormalised).  Ties go to the lower index.
-// One wave per token.  With `x` (a token's input row, activation dtype X) and `router` (fp32 [experts (+ 1), width])
-// the logits are computed here, an fp32 product with 16 experts' sums per lane at a time (launches of a few rows,
-// where the product's own launch and the widening of x cost more than the product).
+// One wave per token.
 // ---------------------------------------------------------------------------------
 #define ROUTE_MAX_EXPERTS 1024
 
-template <typename X>
 __global__ __launch_bounds__(64) void group_topk_kernel(const float* __restrict__ logits, int cols,
-                                                        const X* __restrict__ x, long x_stride,
-                                                        const float* __restrict__ router, int width,
                                                         float* __restrict__ weights, int* __restrict__ ids,
                                                         float* __restrict__ extra_out, int experts, int groups,
                                                         int keep, int topk, float route_scale, int normalize) {
@@ -302,34 +297,9 @@ __global__ __launch_bounds__(64) void group_topk_kernel(const float* __restrict_
   __shared__ float gs[ROUTE_MAX_EXPERTS];
   const long t = blockIdx.x;
   const int lane = threadIdx.x;
-  if (x) {
-    const X* xr = x + t * x_stride;
-    const int ne = experts + (extra_out ? 1 : 0);
-    for (int e0 = 0; e0 < ne; e0 += 16) {
-      float acc[16];
-#pragma unroll
-      for (int j = 0; j < 16; ++j) acc[j] = 0.f;
-      for (int i = lane; i < width; i += 64) {
-        const float xv = Conv<X>::ld(xr + i);
-#pragma unroll
-        for (int j = 0; j < 16; ++j)
-          if (e0 + j < ne) acc[j] = fmaf(xv, router[(long)(e0 + j) * width + i], acc[j]);
-      }
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        float v = acc[j];
-        for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-        if (lane == 0 && e0 + j < ne) {
-          if (e0 + j < experts) s[e0 + j] = sigmoidf(v);
-          else extra_out[t] = sigmoidf(v);
-        }
-      }
-    }
-  } else {
-    const float* z = logits + t * cols;
-    for (int e = lane; e < experts; e += 64) s[e] = sigmoidf(z[e]);
-    if (extra_out && lane == 0) extra_out[t] = sigmoidf(z[experts]);
-  }
+  const float* z = logits + t * cols;
+  for (int e = lane; e < experts; e += 64) s[e] = sigmoidf(z[e]);
+  if (extra_out && lane == 0) extra_out[t] = sigmoidf(z[experts]);
   __syncthreads();
   const int per = experts / groups;
   for (int g = lane; g < groups; g += 64) {
@@ -770,24 +740,13 @@ VPSA_EXPORT int vpsa_glu_clamp(const void* x, long x_stride, void* y, int rows, 
 
 VPSA_EXPORT int vpsa_group_topk(const float* logits, int cols, float* weights, int* ids, float* extra_out,
                                 int tokens, int experts, int groups, int keep, int topk, float route_scale,
-                                int normalize, const void* x, long x_stride, const float* router, int width, int x_dtype,
-                                hipStream_t st) {
-  // x / router: the logits are x . router^T, computed by the kernel (logits is then not read); x_dtype 0 bf16, 1 fp32
+                                int normalize, hipStream_t st) {
   if (tokens <= 0) return 0;
   if (experts > ROUTE_MAX_EXPERTS || groups < 1 || experts % groups || keep < 1 || keep > groups ||
-      topk > experts / groups * keep || (!x && cols < experts + (extra_out ? 1 : 0)) || (x && (!router || width < 1)))
+      topk > experts / groups * keep || cols < experts + (extra_out ? 1 : 0))
     return -1;
-  if (x && x_dtype == 0)
-    group_topk_kernel<bf16_t><<<tokens, 64, 0, st>>>(nullptr, 0, (const bf16_t*)x, x_stride, router, width, weights, ids,
-                                                     extra_out, experts, groups, keep, topk, route_scale, normalize);
-  else if (x && x_dtype == 1)
-    group_topk_kernel<float><<<tokens, 64, 0, st>>>(nullptr, 0, (const float*)x, x_stride, router, width, weights, ids,
-                                                    extra_out, experts, groups, keep, topk, route_scale, normalize);
-  else if (x)
-    return -2;
-  else
-    group_topk_kernel<float><<<tokens, 64, 0, st>>>(logits, cols, nullptr, 0, nullptr, 0, weights, ids, extra_out, experts,
-                                                    groups, keep, topk, route_scale, normalize);
+  hipLaunchKernelGGL(group_topk_kernel, dim3(tokens), dim3(64), 0, st, logits, cols, weights, ids, extra_out,
+                     experts, groups, keep, topk, route_scale, normalize);
   return 0;
 }
 

@@ -225,10 +225,10 @@ class ZetalornModel:
         keys = set()
         for s in self.specs:
             m = s.mixer
-            k = ((2 * m.heads, 2 * m.kv_heads, m.dim, m.vdim) if isinstance(m, DiffAttentionSpec)
-                 else (m.left.heads, m.left.kv_heads, m.left.dim, m.left.vdim))
-            if ops.window_mfma_supported(*k, True):
-                keys.add(k[:2])
+            k = ((2 * m.heads, 2 * m.kv_heads, m.dim, m.vdim, m.chunk) if isinstance(m, DiffAttentionSpec)
+                 else (m.left.heads, m.left.kv_heads, m.left.dim, m.left.vdim, 0))
+            if ops.window_mfma_supported(*k[:4], True):
+                keys.add((k[0], k[1], k[4]))   # heads, key heads, chunk size (0: a window)
         return sorted(keys)
 
     def plan_batch(self, meta: BatchMeta, plan: dict, to_dev) -> None:
@@ -261,7 +261,7 @@ class ZetalornModel:
         meta.row_seq = None
 
     # ------------------------------------------------------------------ mixers
-    def _attend(self, q, pool, cache_off, heads, kv_heads, vdim, window, scale, meta: BatchMeta, **how):
+    def _attend(self, q, pool, cache_off, heads, kv_heads, vdim, window, scale, meta: BatchMeta, chunk=0, **how):
         """The windowed-attention kernels over the decode rows and the prefill rows of the step:
         u fp32 [T, heads, vdim], each head on its own value head."""
         t, nd = q.shape[0], meta.num_decode
@@ -276,7 +276,7 @@ class ZetalornModel:
         if meta.num_prefill_seqs > 0:
             ops.window_attention(q[nd:], pool, cache_off, kv_heads, vdim, meta.pre_block_tables, meta.pre_row_seq,
                                  meta.positions[nd:], window, 0, scale, 0.0, None, out=u[nd:],
-                                 tiles=(meta.pre_win_tiles or {}).get((heads, kv_heads)), own_values=True, **how)
+                                 tiles=(meta.pre_win_tiles or {}).get((heads, kv_heads, chunk)), own_values=True, **how)
         return u.view(t, heads, vdim)
 
     def _attention(self, lw: ZetalornLayer, proj: torch.Tensor, pool, cache_off: int, meta: BatchMeta) -> torch.Tensor:
@@ -287,7 +287,7 @@ class ZetalornModel:
                               cos_sin=lw.cos_sin, rot_dims=m.rot.dims, layout=LAYOUTS[m.rot.layout])
         if m.chunk:
             u = self._attend(q, pool, cache_off, 2 * m.heads, 2 * m.kv_heads, m.vdim, m.chunk, m.scale, meta,
-                             chunked=True, maps=2)
+                             chunk=m.chunk, chunked=True, maps=2)
         else:
             u = self._attend(q, pool, cache_off, 2 * m.heads, 2 * m.kv_heads, m.vdim, 1 << 30, m.scale, meta, maps=2)
         y = ops.diff_heads(u, m.kv_heads, lw.lam, eps, 1.0 - m.diff, self.dtype)
@@ -328,8 +328,8 @@ class ZetalornModel:
         """The mixture's output for rows h, fp32."""
         f: FeedForwardSpec = lw.spec.mlp
         t = h.shape[0]
-        # the logits are a true fp32 product of the rows as they are
-        w, ids, _ = ops.route_group_topk(h, lw.router, f.experts, f.groups, f.keep, f.top, 1.0, normalize=f.norm_topk)
+        logits = F.linear(h.float(), lw.router)  # a true fp32 product
+        w, ids, _ = ops.group_topk(logits, f.experts, f.groups, f.keep, f.top, 1.0, normalize=f.norm_topk)
         out = torch.empty((t, h.shape[1]), dtype=torch.float32, device=h.device)
         if ops.moe_glu_grouped_supported(h, lw.w13, lw.w2):
             ys, pos = ops.moe_glu_grouped(h, lw.w13, lw.w2, ids, f.limit, GLU_ALPHA, GLU_UP_BIAS)

@@ -1338,7 +1338,7 @@ def lora_expand(h, bs, slots, y, r_pad):
 
 # --------------------------------------------------------------------------- latent attention, group routing, fp32 residual
 from .latent import (add_rms_norm, build_latent_tiles, embed_scale, gate_up_glu_clamp, gather_rows, glu_clamp,  # noqa: E402,F401
-                     gate_up_act, gated_add_rms_norm, glu_act, rms_norm_add, route_group_topk, route_softmax,
+                     gate_up_act, gated_add_rms_norm, glu_act, rms_norm_add, route_softmax,
                      group_topk, latent_attention, moe_glu_grouped, moe_glu_grouped_supported, up_relu_sq,
                      latent_kv_write, latent_mfma_supported, latent_tile_kernel_takes, moe_finish, relu_sq, rms_norm_rows, rope_pairs, sigmoid_gate)
 

@@ -389,33 +389,7 @@ def group_topk(logits, experts: int, groups: int, keep: int, topk: int, route_sc
     ex = torch.empty((t,), dtype=torch.float32, device=logits.device) if extra else None
     o._check(o._kernels().vpsa_group_topk(o._p(logits), c_int(logits.shape[1]), o._p(w), o._p(ids), o._p(ex), c_int(t),
                                           c_int(experts), c_int(groups), c_int(keep), c_int(topk),
-                                          c_float(route_scale), c_int(1 if normalize else 0), None, c_long(0), None,
-                                          c_int(0), c_int(0), o._stream()), "group_topk")
-    return w, ids, ex
-
-
-ROUTE_FUSED_MAX_ROWS = 256   # up to here the routing kernel computes the logits itself
-
-
-def route_group_topk(h, router, experts: int, groups: int, keep: int, topk: int, route_scale: float, extra: bool = False,
-                     normalize: bool = False):
-    """``group_topk`` of the logits ``h @ router.T`` (h [T, width] in the activation dtype, router fp32
-    [experts (+ 1), width]; an fp32 product of the rows as they are).  Launches of a few rows compute the logits inside
-    the routing kernel; larger ones through the library's fp32 product."""
-    if not h.is_cuda or h.shape[0] > ROUTE_FUSED_MAX_ROWS:
-        logits = torch.nn.functional.linear(h.float(), router)
-        return group_topk(logits, experts, groups, keep, topk, route_scale, extra, normalize)
-    o = _ops()
-    _f32(router)
-    t, width = h.shape
-    assert _rows(h) and router.shape == (experts + (1 if extra else 0), width)
-    w = torch.empty((t, topk), dtype=torch.float32, device=h.device)
-    ids = torch.empty((t, topk), dtype=torch.int32, device=h.device)
-    ex = torch.empty((t,), dtype=torch.float32, device=h.device) if extra else None
-    o._check(o._kernels().vpsa_group_topk(None, c_int(0), o._p(w), o._p(ids), o._p(ex), c_int(t), c_int(experts),
-                                          c_int(groups), c_int(keep), c_int(topk), c_float(route_scale),
-                                          c_int(1 if normalize else 0), o._p(h), c_long(h.stride(0)), o._p(router),
-                                          c_int(width), c_int(_dt(h)), o._stream()), "route_group_topk")
+                                          c_float(route_scale), c_int(1 if normalize else 0), o._stream()), "group_topk")
     return w, ids, ex
 
 

@@ -435,10 +435,11 @@ def window_mfma_supported(heads: int, kv_heads: int, dim: int, vdim: int, own_va
                                                              c_int(1 if own_values else 0)))
 
 
-def build_window_tiles(q_lens, ctx_lens, heads: int, kv_heads: int):
+def build_window_tiles(q_lens, ctx_lens, heads: int, kv_heads: int, chunk: int = 0):
     """Work list of the matrix-core kernel for the prefill part of a batch: int32 rows (sequence, first
     query row, rows, position of the first row); a tile holds consecutive rows of one sequence, as many as
-    fit the kernel's slots ((row, query head of one KV group) pairs).  Latest rows first (they visit the most pages)."""
+    fit the kernel's slots ((row, query head of one KV group) pairs).  Latest rows first (they visit the most pages);
+    with ``chunk`` (rows that see their own chunk of positions only) the rows deepest into their chunk first."""
     import numpy as np
 
     per = max(1, window_tile_slots() // (heads // kv_heads))
@@ -451,7 +452,8 @@ def build_window_tiles(q_lens, ctx_lens, heads: int, kv_heads: int):
     if not parts:
         return np.zeros((0, 4), dtype=np.int32)
     tiles = np.concatenate(parts)
-    return tiles[np.argsort(-tiles[:, 3], kind="stable")].astype(np.int32)
+    work = tiles[:, 3] % chunk if chunk else tiles[:, 3]
+    return tiles[np.argsort(-work, kind="stable")].astype(np.int32)
 
 
 def window_decode_splits(rows: int, kv_heads: int, window: int, keep_first: int, max_ctx: int) -> int:
