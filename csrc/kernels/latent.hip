@@ -620,9 +620,22 @@ __global__ __launch_bounds__(256) void moe_finish_kernel(float* __restrict__ res
   // overwrite: the sum replaces what `residual` held (a buffer of its own instead of a stream)
   const long t = blockIdx.x;
   const float sg = shared ? (gate ? gate[t] : 1.f) : 0.f;
+  // the first pairs' weights and rows are read once, ahead of the walk over the channels (a launch of a few
+  // tokens is bound by the chain weight -> row index -> value, not by bytes)
+  constexpr int AHEAD = 8;
+  float wk[AHEAD];
+  const T* yk[AHEAD];
+#pragma unroll
+  for (int k = 0; k < AHEAD; ++k) {
+    wk[k] = k < topk ? weights[t * topk + k] : 0.f;
+    yk[k] = y + (long)(wk[k] != 0.f ? pos[t * topk + k] : 0) * n;
+  }
   for (int i = threadIdx.x; i < n; i += 256) {
     float a = 0.f;
-    for (int k = 0; k < topk; ++k) {
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k)
+      if (wk[k] != 0.f) a += wk[k] * Conv<T>::ld(yk[k] + i);
+    for (int k = AHEAD; k < topk; ++k) {
       const float w = weights[t * topk + k];
       if (w != 0.f) a += w * Conv<T>::ld(y + (long)pos[t * topk + k] * n + i);
     }

@@ -896,7 +896,7 @@ def zetalorn_stack(width, heads, experts, unit_ff, top, blocks=1):
 # two layers run twice
 PRESETS["tiny-zetalorn"] = zetalorn_config(
     "tiny-zetalorn", 512, 128,
-    [_zx_parallel(4, 2, 64, 128, 96, 8, 2, 32, 64, _zx_moe(64, 6, 2, 2, 1)),
+    [_zx_parallel(4, 2, 64, 128, 80, 8, 2, 32, 64, _zx_moe(64, 6, 2, 2, 1)),
      _zx_attention(4, 2, 64, 128, 160, _zx_moe(64, 4, 2, 1, 1)),
      _zx_parallel(2, 1, 64, 128, 64, 16, 2, 64, 32)], loop={"start": 0, "stop": 2, "times": 2}, logit_scale=0.5,
     max_position_embeddings=4096)
