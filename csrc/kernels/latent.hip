@@ -18,6 +18,7 @@
 //   route_softmax      softmax scores (+ a selection bias) -> best groups by their largest biased score -> top-k;
 //                      trailing identity experts leave the pair list and come back as one gate per token
 //   rmsnorm_add        residual += rmsnorm(delta) * w;  y = residual (activation dtype)
+//   gated_add_rmsnorm  residual += sigmoid(gate + b) (.) (c1 n1(d1) + c2 n2(d2)) + extra + vector;  y = rmsnorm(residual) w
 //   glu_act            silu(g) * u  or  gelu_tanh(g) * u  of  x = g | u
 //   gather_rows        xs[r] = x[idx[r]]
 //   moe_finish         residual[t] += sum_k w[t,k] * y[pos[t,k]] + gate[t] * shared[t]

@@ -7,17 +7,24 @@
 //
 //   add_dyt            residual += s1 d1 + s2 d2;  y = tanh(alpha residual) w + b
 //   recurrent_scan     per (sequence, head): S <- a_t (.) S + k_t v_t^T,  o_t = S^T q_t, state in registers,
-//                      carried in a per-sequence fp32 slot (zero when the chunk starts at position 0)
+//                      carried in a per-sequence fp32 slot (zero when the chunk starts at position 0); the fixed-decay
+//                      form optionally on silu(q), silu(k), silu(v)
 //   head_rms           o[t, h, :] / rms(o[t, h, :]) (* w) (* silu(gate[t, h, :]))
 //   short_conv_qkv     y_t = sum_j w[:, j] u_(t - taps + 1 + j) over a sequence's projected rows (the rows
 //                      before the chunk come from the sequence's slot), rotary q / k, k and v -> paged cache
 //   conv_tail          the last taps - 1 projected rows of every sequence -> its slot
 //   window_attention   softmax(cap tanh(q k scale / cap)) with a sink in the denominator over the keys
-//                      j <= i with i - j < window or j < keep_first, applied to the values of EVERY KV head
+//                      j <= i with i - j < window or j < keep_first (or: of i's own chunk of positions; or: of the
+//                      window and one pooled entry per block of tokens before it), applied to the values of EVERY
+//                      KV head or of the head's own
 //   mix_heads          out[t, h] = sum_g talk[h, g] u[t, g, kv_head(h)]
 //   xielu              z > 0: a_p z^2 + z / 2;  else a_n (exp(z) - 1 - z) + z / 2
-//   qk_norm_write      q and k heads to unit root mean square (no weight), q times a temperature that grows with
-//                      the logarithm of the position, k and v -> paged cache (the layout window_attention reads)
+//   qk_norm_write      q and k heads to unit root mean square (a weight per channel, a rotation of the first
+//                      channels where given), q times a temperature that grows with the logarithm of the position,
+//                      k and v -> paged cache (the layout window_attention reads; value heads may be fewer than key heads)
+//   pool_blocks        mean key and mean value of every block of P tokens a step completes -> the pooled region of
+//                      the sequence's pages (window_attention with pool > 0 sees the blocks before its window)
+//   diff_heads         a1 - lambda a2 of a differential attention's two maps, unit root mean square, a factor
 //   gla_prepare        q scale | k | sigmoid(z + b)^(1 / tau) per key channel, for prepared_scan
 //   mlstm_gates        capped exponential input / forget gates of a matrix memory with their running maximum
 //                      (carried per sequence and head), turned into one decay and one write strength per token
@@ -25,7 +32,8 @@
 //   prepared_scan      recurrent_scan on rows prepared by the caller; optionally one more value column of ones,
 //                      whose read-out is the normaliser's dot product with the query
 //   head_finish        head_rms with its parts optional: stabilised division by the normaliser column, unit RMS,
-//                      a weight per channel or per head and channel, a silu or sigmoid gate
+//                      a weight per channel or per head and channel, a silu or sigmoid gate (a workgroup per head
+//                      from a thousand channels on)
 //
 // Plain kernels: every size is taken (bounds below are checked by the entry points).
 #include "common.h"

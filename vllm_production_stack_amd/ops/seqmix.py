@@ -8,7 +8,8 @@ Two stores, both owned by the engine's runner:
 
 - the paged pool ``[pages, page_elems]`` (activation dtype): a layer with windowed attention keeps, per
   page and ``cache_off`` elements into it, ``K [PAGE, kv_heads * dim]`` then V transposed,
-  ``[kv_heads * vdim, PAGE]`` (a channel's 64 keys are contiguous);
+  ``[kv_heads * vdim, PAGE]`` (a channel's 64 keys are contiguous); a layer that also sees pooled blocks of
+  tokens keeps a second region of the same shape behind it for the blocks' mean keys and values;
 - the state pool ``[slots, state_elems]`` (fp32): a sequence's slot holds, per layer and ``state_off``
   elements into it, a recurrence's ``[heads, dim, vdim]`` matrix or the ``conv - 1`` projected rows
   a convolution still needs.  A chunk that starts at position 0 starts from zeros, whatever the slot
