@@ -43,6 +43,7 @@ def _kernels():
             "vpsa_moe_mfma_act",
             "vpsa_add_dyt", "vpsa_recurrent_scan", "vpsa_head_rms", "vpsa_short_conv_qkv", "vpsa_window_attention",
             "vpsa_mix_heads", "vpsa_xielu", "vpsa_window_mfma_supported", "vpsa_window_attention_mfma", "vpsa_window_tile_slots",
+            "vpsa_gated_add_rmsnorm", "vpsa_pool_blocks", "vpsa_diff_heads",
         ):
             getattr(lib, name).restype = c_int
         lib.vpsa_prefill_split_record_bytes.restype = c_long
