@@ -3,7 +3,6 @@ against the float64 oracle.  The CPU and the GPU test files call them with their
 
 from __future__ import annotations
 
-import math
 import tempfile
 
 import torch
